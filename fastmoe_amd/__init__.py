@@ -1,0 +1,24 @@
+r"""fastmoe_amd: the single-GPU MoE-layer hot path of FastMoE, native to MI355X.
+
+`FMoE`, `FMoELinear`, `FMoETransformerMLP` and the gates keep the reference's
+interface; `fmoe_cuda` is the operator module that stands in for the
+reference's compiled extension of the same name.
+"""
+from . import fmoe_cuda
+from .gates import BaseGate, GShardGate, NaiveGate, SwitchGate
+from .layers import FMoE
+from .linear import FMoELinear
+from .transformer import FMoETransformerMLP
+
+
+def install_as_fmoe_cuda() -> None:
+    """Registers the operator module as `fmoe_cuda`, so that the reference's
+    own Python package (`import fmoe_cuda` in fmoe/functions.py:9) binds to the
+    MI355X kernels."""
+    import sys
+
+    sys.modules.setdefault("fmoe_cuda", fmoe_cuda)
+
+
+__all__ = ["FMoE", "FMoELinear", "FMoETransformerMLP", "BaseGate", "NaiveGate",
+           "GShardGate", "SwitchGate", "fmoe_cuda", "install_as_fmoe_cuda"]

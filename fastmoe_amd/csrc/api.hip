@@ -1,0 +1,200 @@
+// C ABI glue: error text, the expert-linear entry points (kernel selection,
+// bias gradient) and the host-count upload.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "gemm.h"
+
+namespace fmoe {
+
+static thread_local char g_err[512] = "";
+static int g_gemm_path = 0;  // 0 = automatic, 1 = scalar kernel only
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// ------------------------------------------------------------ bias gradient
+// db[e][c] = sum over the rows of expert e of dy[r][c], fp32 accumulation
+// (fp64 for doubles).  Block = 32 column groups x 8 row lanes; a thread adds
+// VEC adjacent columns of every 8th row, then the 8 row lanes meet in LDS.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bias_grad_kernel(
+    const T* __restrict__ dy, const int32_t* __restrict__ seg_off,
+    T* __restrict__ db, int out_feat) {
+  using acc_t = typename Elem<T>::acc_t;
+  struct alignas(sizeof(T) * VEC) Pk { T v[VEC]; };
+  __shared__ acc_t part[8][32 * VEC + 1];
+  const int e = blockIdx.y;
+  const int cx = threadIdx.x % 32, ry = threadIdx.x / 32;
+  const int c0 = (blockIdx.x * 32 + cx) * VEC;
+  const int r_begin = seg_off[e], r_end = seg_off[e + 1];
+  acc_t acc[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) acc[v] = 0;
+  if (c0 < out_feat) {
+    for (int r = r_begin + ry; r < r_end; r += 8) {
+      const Pk p = *reinterpret_cast<const Pk*>(dy + (int64_t)r * out_feat + c0);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) acc[v] += Elem<T>::to_acc(p.v[v]);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) part[ry][cx * VEC + v] = acc[v];
+  __syncthreads();
+  for (int c = threadIdx.x; c < 32 * VEC; c += 256) {
+    acc_t s = 0;
+#pragma unroll
+    for (int y = 0; y < 8; ++y) s += part[y][c];
+    const int col = blockIdx.x * 32 * VEC + c;
+    if (col < out_feat) db[(int64_t)e * out_feat + col] = Elem<T>::from_acc(s);
+  }
+}
+
+template <typename T>
+static int launch_bias_grad(const void* dy, const int32_t* seg_off, void* db,
+                            int out_feat, int n_expert, hipStream_t s) {
+  constexpr int kVec = 16 / sizeof(T);
+  const bool vec = out_feat % kVec == 0 && ((uintptr_t)dy % 16) == 0;
+  if (vec) {
+    dim3 grid(ceil_div(out_feat, 32 * kVec), n_expert);
+    hipLaunchKernelGGL((bias_grad_kernel<T, kVec>), grid, dim3(256), 0, s,
+                       (const T*)dy, seg_off, (T*)db, out_feat);
+  } else {
+    dim3 grid(ceil_div(out_feat, 32), n_expert);
+    hipLaunchKernelGGL((bias_grad_kernel<T, 1>), grid, dim3(256), 0, s,
+                       (const T*)dy, seg_off, (T*)db, out_feat);
+  }
+  FMOE_LAUNCH_CHECK("bias_grad");
+  return FMOE_OK;
+}
+
+// ------------------------------------------------------- host-count upload
+struct OffChunk { int32_t v[512]; };
+__global__ void write_offsets_kernel(OffChunk c, int32_t* dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = c.v[i];
+}
+
+static int check_linear(const char* who, int64_t n_rows, int64_t in_feat,
+                        int64_t out_feat, int64_t n_expert, int dtype) {
+  FMOE_REQUIRE(dtype_size(dtype) != 0, FMOE_ERR_INVALID, "%s: unknown dtype %d",
+               who, dtype);
+  FMOE_REQUIRE(n_rows >= 0 && in_feat >= 1 && out_feat >= 1 && n_expert >= 1,
+               FMOE_ERR_INVALID,
+               "%s: bad sizes rows=%lld in=%lld out=%lld experts=%lld", who,
+               (long long)n_rows, (long long)in_feat, (long long)out_feat,
+               (long long)n_expert);
+  FMOE_REQUIRE(n_rows < ((int64_t)1 << 31) && in_feat < ((int64_t)1 << 31) &&
+                   out_feat < ((int64_t)1 << 31) && n_expert <= 65535,
+               FMOE_ERR_UNSUPPORTED, "%s: size exceeds the int32 index range", who);
+  return FMOE_OK;
+}
+
+static int run_gemm(int mode, const GemmArgs& g, int dtype, hipStream_t s) {
+  if (g_gemm_path == 0 && gemm_mfma_supported(mode, g, dtype))
+    return launch_gemm_mfma(mode, g, dtype, s);
+  return launch_gemm_simt(mode, g, dtype, s);
+}
+
+}  // namespace fmoe
+
+using namespace fmoe;
+
+extern "C" const char* fmoe_version(void) { return "fastmoe_amd 0.1 (gfx950)"; }
+extern "C" const char* fmoe_last_error(void) { return g_err; }
+
+extern "C" int fmoe_set_gemm_path(int path) {
+  FMOE_REQUIRE(path == 0 || path == 1, FMOE_ERR_INVALID, "gemm path must be 0 or 1");
+  g_gemm_path = path;
+  return FMOE_OK;
+}
+
+extern "C" int fmoe_seg_off_from_host_counts(const int64_t* expert_count_host,
+                                             int64_t n_expert, int32_t* seg_off,
+                                             void* stream) {
+  FMOE_REQUIRE(expert_count_host && seg_off && n_expert >= 1, FMOE_ERR_INVALID,
+               "seg_off_from_host_counts: bad arguments");
+  hipStream_t s = (hipStream_t)stream;
+  // offsets travel as kernel arguments: no staging copy, nothing to keep alive
+  int64_t run = 0;
+  int64_t done = 0;  // entries of seg_off already written
+  OffChunk chunk;
+  int fill = 0;
+  for (int64_t e = 0; e <= n_expert; ++e) {
+    FMOE_REQUIRE(run >= 0 && run < ((int64_t)1 << 31), FMOE_ERR_INVALID,
+                 "seg_off_from_host_counts: counts negative or too large");
+    chunk.v[fill++] = (int32_t)run;
+    if (e < n_expert) {
+      FMOE_REQUIRE(expert_count_host[e] >= 0, FMOE_ERR_INVALID,
+                   "seg_off_from_host_counts: negative count for expert %lld",
+                   (long long)e);
+      run += expert_count_host[e];
+    }
+    if (fill == 512 || e == n_expert) {
+      hipLaunchKernelGGL(write_offsets_kernel, dim3(2), dim3(256), 0, s, chunk,
+                         seg_off + done, fill);
+      FMOE_LAUNCH_CHECK("write_offsets");
+      done += fill;
+      fill = 0;
+    }
+  }
+  return FMOE_OK;
+}
+
+extern "C" int fmoe_grouped_linear_fwd(const void* x, const void* w,
+                                       const void* bias, const int32_t* seg_off,
+                                       void* y, int64_t n_rows, int64_t in_feat,
+                                       int64_t out_feat, int64_t n_expert,
+                                       int dtype, void* stream) {
+  int rc = check_linear("grouped_linear_fwd", n_rows, in_feat, out_feat, n_expert, dtype);
+  if (rc) return rc;
+  if (n_rows == 0) return FMOE_OK;
+  FMOE_REQUIRE(x && w && seg_off && y, FMOE_ERR_INVALID,
+               "grouped_linear_fwd: null pointer");
+  GemmArgs g{x, w, y, bias, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert};
+  return run_gemm(GEMM_FWD, g, dtype, (hipStream_t)stream);
+}
+
+extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
+                                       const void* w, const int32_t* seg_off,
+                                       void* dx, void* dw, void* dbias,
+                                       int64_t n_rows, int64_t in_feat,
+                                       int64_t out_feat, int64_t n_expert,
+                                       int dtype, void* stream) {
+  int rc = check_linear("grouped_linear_bwd", n_rows, in_feat, out_feat, n_expert, dtype);
+  if (rc) return rc;
+  FMOE_REQUIRE(seg_off != nullptr, FMOE_ERR_INVALID,
+               "grouped_linear_bwd: seg_off is null");
+  FMOE_REQUIRE(n_rows == 0 || dy != nullptr, FMOE_ERR_INVALID,
+               "grouped_linear_bwd: dy is null");
+  hipStream_t s = (hipStream_t)stream;
+  if (dx && n_rows > 0) {
+    FMOE_REQUIRE(w != nullptr, FMOE_ERR_INVALID, "grouped_linear_bwd: w is null");
+    GemmArgs g{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert};
+    rc = run_gemm(GEMM_DGRAD, g, dtype, s);
+    if (rc) return rc;
+  }
+  if (dw) {
+    // runs also for n_rows == 0: experts without rows get zero gradients
+    FMOE_REQUIRE(n_rows == 0 || x != nullptr, FMOE_ERR_INVALID,
+                 "grouped_linear_bwd: x is null");
+    GemmArgs g{dy, x, dw, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert};
+    rc = run_gemm(GEMM_WGRAD, g, dtype, s);
+    if (rc) return rc;
+  }
+  if (dbias) {
+    switch (dtype) {
+      case FMOE_F32: rc = launch_bias_grad<float>(dy, seg_off, dbias, (int)out_feat, (int)n_expert, s); break;
+      case FMOE_F64: rc = launch_bias_grad<double>(dy, seg_off, dbias, (int)out_feat, (int)n_expert, s); break;
+      case FMOE_F16: rc = launch_bias_grad<__half>(dy, seg_off, dbias, (int)out_feat, (int)n_expert, s); break;
+      default: rc = launch_bias_grad<__hip_bfloat16>(dy, seg_off, dbias, (int)out_feat, (int)n_expert, s); break;
+    }
+    if (rc) return rc;
+  }
+  return FMOE_OK;
+}

@@ -1,0 +1,43 @@
+// Shared declarations of the grouped expert GEMMs (one launch for all experts).
+#pragma once
+#include "common.h"
+
+namespace fmoe {
+
+// The three products of an expert linear layer, all over the rows
+// [seg_off[e], seg_off[e+1]) of expert e:
+//   FWD    Y[seg]  = X[seg]  * W_e^T (+ b_e)   M = rows, N = out,  K = in
+//   DGRAD  dX[seg] = dY[seg] * W_e             M = rows, N = in,   K = out
+//   WGRAD  dW_e    = dY[seg]^T * X[seg]        M = out,  N = in,   K = rows
+enum GemmMode { GEMM_FWD = 0, GEMM_DGRAD = 1, GEMM_WGRAD = 2 };
+
+struct GemmArgs {
+  const void* a;        // FWD: x      DGRAD: dy     WGRAD: dy
+  const void* b;        // FWD: w      DGRAD: w      WGRAD: x
+  void* c;              // FWD: y      DGRAD: dx     WGRAD: dw
+  const void* bias;     // FWD only, may be null
+  const int32_t* seg_off;
+  int64_t n_rows;       // rows allocated in the row-major activations
+  int in_feat;
+  int out_feat;
+  int n_expert;
+};
+
+// Virtual row-tile index space for the ragged products: expert e owns the
+// tiles [seg_off[e] / BM + e, ... + ceil(cnt_e / BM)); the starts are strictly
+// increasing in e, so no prefix sum over tile counts is needed and tiles that
+// belong to nobody simply exit.
+inline int virtual_row_tiles(int64_t n_rows, int n_expert, int bm) {
+  return (int)(n_rows / bm) + n_expert;
+}
+
+// Scalar (non-matrix-core) grouped GEMM for any dtype and any shape.
+int launch_gemm_simt(int mode, const GemmArgs& g, int dtype, hipStream_t s);
+
+// bf16 / f16 grouped GEMM on the matrix cores.  Returns FMOE_ERR_UNSUPPORTED
+// without launching when the shape does not fit (callers then use the scalar
+// kernel).
+bool gemm_mfma_supported(int mode, const GemmArgs& g, int dtype);
+int launch_gemm_mfma(int mode, const GemmArgs& g, int dtype, hipStream_t s);
+
+}  // namespace fmoe

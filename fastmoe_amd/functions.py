@@ -1,0 +1,184 @@
+r"""Autograd functions of the MoE dispatch, mirroring fmoe/functions.py of the
+reference (same names and argument lists), plus the fused variants this
+package's own layer uses: they keep every count on the device, so a forward
+pass needs no device-to-host copy.
+"""
+from __future__ import annotations
+
+import torch
+from torch.autograd import Function
+
+from . import fmoe_cuda
+
+
+# --------------------------------------------------------------------------
+# Reference-shaped helpers (fmoe/functions.py:28-193), world_size == 1 only
+# --------------------------------------------------------------------------
+def _single_worker(world_size):
+    if world_size != 1:
+        raise NotImplementedError(
+            "this build covers the single-GPU path (world_size == 1); "
+            "expert exchange across workers is out of scope")
+
+
+def count_by_gate(gate, num_expert, world_size, require_pos=True):
+    """(pos, local_expert_count, global_expert_count) as fmoe/functions.py:28-49
+    returns them: pos int64[N_valid] on the device (None if not required), the
+    counts int64[E] on the device (one tensor for both at world_size 1).
+
+    Without positions this is one histogram launch; with them, one fused
+    routing call plus the single host read that sizes `pos`."""
+    _single_worker(world_size)
+    gate = gate.contiguous()
+    with torch.no_grad():
+        if not require_pos:
+            hist = torch.zeros(num_expert, device=gate.device, dtype=torch.int32)
+            fmoe_cuda.expert_count(gate, hist)
+            counts = hist.long()
+            return None, counts, counts
+        pos, counts, seg_off, _ = fmoe_cuda.route(gate, num_expert, want_inv=False)
+        n_valid = int(seg_off[-1].item())
+    return pos[:n_valid], counts, counts
+
+
+def prepare_forward(gate, num_expert, world_size):
+    """(pos, local_expert_count, global_expert_count, fwd_expert_count,
+    fwd_batch_size) with the three counts on the host, as
+    fmoe/functions.py:52-75 hands them to the dispatch."""
+    pos, counts, _ = count_by_gate(gate, num_expert, world_size)
+    host = counts.cpu()
+    return pos, host, host, host.clone(), int(host.sum())
+
+
+def _local_scatter(inp, pos):
+    return fmoe_cuda.local_scatter(inp.contiguous(), pos)
+
+
+def _local_gather(inp, pos, out_batch_size, maybe_overlap=True):
+    return fmoe_cuda.local_gather(inp.contiguous(), pos, out_batch_size,
+                                  maybe_overlap)
+
+
+class MOEScatter(Function):
+    r"""Rows of `inp` gathered into expert order; fmoe/functions.py:93-142."""
+
+    @staticmethod
+    def forward(ctx, inp, pos, local_expert_count, global_expert_count,
+                fwd_batch_size, world_size):
+        _single_worker(world_size)
+        local_input_buf = _local_scatter(inp, pos)
+        ctx.moe_args = inp.shape[0], pos.shape[0], world_size
+        ctx.save_for_backward(pos, local_expert_count, global_expert_count)
+        return local_input_buf
+
+    @staticmethod
+    def backward(ctx, global_grad_in):
+        (pos, _lec, _gec) = ctx.saved_tensors
+        (inp_batch_size, _buf_batch_size, _world_size) = ctx.moe_args
+        grad_in = _local_gather(global_grad_in, pos, inp_batch_size)
+        return grad_in, None, None, None, None, None
+
+
+class MOEGather(Function):
+    r"""Expert-ordered rows put back at their slots; fmoe/functions.py:144-193."""
+
+    @staticmethod
+    def forward(ctx, global_output_buf, pos, local_expert_count,
+                global_expert_count, local_batch_size, world_size):
+        _single_worker(world_size)
+        output = _local_gather(global_output_buf, pos, local_batch_size,
+                               maybe_overlap=False)
+        ctx.moe_args = (global_output_buf.shape[0], world_size)
+        ctx.save_for_backward(pos, local_expert_count, global_expert_count)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        pos, _lec, _gec = ctx.saved_tensors
+        grad_out_buf = _local_scatter(grad_out.contiguous(), pos)
+        return grad_out_buf, None, None, None, None, None
+
+
+# --------------------------------------------------------------------------
+# Fused, synchronisation-free path
+# --------------------------------------------------------------------------
+class SegmentTable:
+    """Per-expert row segments kept on the device.
+
+    seg_off  int32[E+1]  exclusive prefix of the row counts
+    counts   int64[E]    rows per expert (what the reference calls
+                         fwd_expert_count, fmoe/functions.py:66-67)
+    """
+
+    def __init__(self, seg_off: torch.Tensor, counts: torch.Tensor):
+        self.seg_off = seg_off
+        self.counts = counts
+        self._host = None
+
+    @property
+    def num_expert(self) -> int:
+        return self.counts.numel()
+
+    def cpu(self) -> torch.Tensor:
+        """Host int64 counts (one device-to-host copy, cached)."""
+        if self._host is None:
+            self._host = self.counts.cpu()
+        return self._host
+
+
+class RoutePlan:
+    """Everything the dispatch needs about one routing decision."""
+
+    def __init__(self, gate: torch.Tensor, num_expert: int):
+        self.top_k = gate.shape[1] if gate.dim() == 2 else 1
+        self.n_tokens = gate.shape[0]
+        self.n_slots = gate.numel()
+        with torch.no_grad():
+            pos, counts, seg_off, inv = fmoe_cuda.route(gate.contiguous(), num_expert)
+        self.pos = pos
+        self.inv = inv
+        self.segments = SegmentTable(seg_off, counts)
+
+    @property
+    def n_rows_dev(self) -> torch.Tensor:
+        """Device int32 holding the number of live rows (= seg_off[E])."""
+        return self.segments.seg_off[-1:]
+
+
+class FusedScatter(Function):
+    r"""buf[r] = inp[pos[r] // k]; backward sums a token's k rows in a fixed
+    order (no float atomics).  Replaces MOEScatter at world_size 1."""
+
+    @staticmethod
+    def forward(ctx, inp, plan: RoutePlan):
+        ctx.plan = plan
+        return fmoe_cuda.local_scatter(inp.contiguous(), plan.pos, plan.top_k,
+                                       plan.n_rows_dev)
+
+    @staticmethod
+    def backward(ctx, grad_buf):
+        plan = ctx.plan
+        return fmoe_cuda.scatter_reduce(grad_buf.contiguous(), plan.inv,
+                                        plan.n_tokens, plan.top_k), None
+
+
+class FusedGatherCombine(Function):
+    r"""y[t] = sum_j score[t, j] * buf[row of slot (t, j)]: MOEGather followed
+    by the bmm of fmoe/layers.py:288-295 in one pass over the rows."""
+
+    @staticmethod
+    def forward(ctx, buf, score, plan: RoutePlan):
+        buf = buf.contiguous()
+        score = score.contiguous().to(buf.dtype)
+        ctx.plan = plan
+        ctx.save_for_backward(buf, score)
+        return fmoe_cuda.gather_combine_fwd(buf, plan.inv, score, plan.n_tokens,
+                                            plan.top_k)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        buf, score = ctx.saved_tensors
+        plan = ctx.plan
+        dbuf, dscore = fmoe_cuda.gather_combine_bwd(
+            grad_y.contiguous(), buf, plan.inv, score, plan.n_tokens, plan.top_k)
+        return dbuf, dscore.view_as(score), None

@@ -1,0 +1,28 @@
+r"""Top-k of a linear layer (fmoe/gates/naive_gate.py)."""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .base_gate import BaseGate
+
+
+class NaiveGate(BaseGate):
+    r"""logits = Linear(d_model, experts); the k largest logits pick the experts
+    and their softmax gives the combine weights.  Returns `(idx [T, k] int64,
+    score [T, k])`, plus the full logits when `return_all_scores`."""
+
+    def __init__(self, d_model, num_expert, world_size, top_k=2, gate_bias=True):
+        super().__init__(num_expert, world_size)
+        self.gate = nn.Linear(d_model, self.tot_expert, bias=gate_bias)
+        self.top_k = top_k
+
+    def forward(self, inp, return_all_scores=False):
+        logits = self.gate(inp)
+        top_val, top_idx = torch.topk(logits, k=self.top_k, dim=-1, largest=True,
+                                      sorted=False)
+        score = F.softmax(top_val.view(-1, self.top_k), dim=-1)
+        # a zero loss so training loops can always call get_loss()
+        self.set_loss(torch.zeros(1, requires_grad=True).to(inp.device))
+        if return_all_scores:
+            return top_idx, score, logits
+        return top_idx, score

@@ -1,0 +1,237 @@
+/*
+ * fmoe_hip.h -- C ABI of the MI355X (gfx950) single-GPU MoE-layer hot path.
+ *
+ * Every entry point is `extern "C"`, takes plain device pointers, sizes and a
+ * HIP stream (as void*), launches asynchronously on that stream and returns 0
+ * or a negative fmoe_status.  Nothing here exits the process; the text of the
+ * last failure on the calling thread is available from fmoe_last_error().
+ *
+ * Citations name the interface of the reference (laekov/fastmoe) that each
+ * entry point stands in for, as path:line in the reference tree.
+ *
+ * Conventions
+ *   gate / pos      int64, as produced by torch.topk and consumed by the
+ *                   reference's Python (fmoe/functions.py:28-49).
+ *   counts          int32 for histograms and capacities (cuda/balancing.cu:6-8),
+ *                   int64 where the reference hands them to Python.
+ *   slots           the N = tokens * top_k routed entries of `gate`, flat index
+ *                   i = token * top_k + j.
+ *   rows            the N_valid slots that survived (gate != -1), grouped by
+ *                   expert; row r of a dispatch buffer holds slot pos[r].
+ *   seg_off         int32[E+1] exclusive prefix of per-expert row counts;
+ *                   expert e owns rows [seg_off[e], seg_off[e+1]).
+ *   inv             int32[N]: inv[pos[r]] = r, and -1 for dropped slots.
+ *   order           rows of one expert are in ascending slot index (stable),
+ *                   which is one legal outcome of the reference's atomics.
+ */
+#ifndef FMOE_HIP_H_
+#define FMOE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum fmoe_status {
+  FMOE_OK = 0,
+  FMOE_ERR_INVALID = -1,     /* bad argument (null pointer, negative size, ...) */
+  FMOE_ERR_UNSUPPORTED = -2, /* shape / dtype outside what the kernels handle   */
+  FMOE_ERR_HIP = -3,         /* a HIP runtime call or a launch failed           */
+  FMOE_ERR_WORKSPACE = -4    /* workspace missing or too small                  */
+} fmoe_status;
+
+typedef enum fmoe_dtype {
+  FMOE_F32 = 0,
+  FMOE_F64 = 1,
+  FMOE_F16 = 2,
+  FMOE_BF16 = 3
+} fmoe_dtype;
+
+/* Largest number of experts the routing kernels keep in LDS. */
+#define FMOE_MAX_EXPERTS 4096
+
+/* Library identification and error text (thread-local, never NULL). */
+const char* fmoe_version(void);
+const char* fmoe_last_error(void);
+
+/* ------------------------------------------------------------------ routing */
+
+/*
+ * Histogram of gate indices: expert_count[e] += #{i : gate_idx[i] == e}.
+ * Entries equal to -1 or outside [0, n_expert) are skipped; the output is
+ * accumulated into, not overwritten (the caller zero-fills).
+ * Replaces fmoe_cuda.expert_count: cuda/fmoe_cuda.cpp:43-45,
+ * cuda/local_exchange.cu:22-32, kernel cuda/local_exchange.cuh:36-78.
+ */
+int fmoe_expert_count(const int64_t* gate_idx, int64_t numel,
+                      int32_t* expert_count, int32_t n_expert, void* stream);
+
+/*
+ * Bytes of device workspace needed by fmoe_assign_pos, fmoe_route and
+ * fmoe_prune_gate_by_capacity for `numel` slots and `n_expert` experts.
+ * Returns a negative fmoe_status on bad arguments.
+ */
+int64_t fmoe_route_workspace_bytes(int64_t numel, int32_t n_expert);
+
+/*
+ * Positions from an inclusive cumulative count.
+ * In:  cum_count[e] = sum_{e'<=e} count[e'] (int32), gate (int64, numel slots).
+ * Out: pos[off[e] .. cum_count[e]) = the slots routed to e in ascending slot
+ *      index, off[e] = cum_count[e] - count[e].  On return cum_count[e] = off[e],
+ *      the state the reference's atomicSub leaves behind.
+ * Replaces fmoe_cuda.assign_pos: cuda/fmoe_cuda.cpp:39-42,
+ * cuda/local_exchange.cu:5-20, kernel cuda/local_exchange.cuh:5-26.
+ */
+int fmoe_assign_pos(int32_t* cum_count, const int64_t* gate, int64_t* pos,
+                    int64_t numel, int32_t n_expert, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+
+/*
+ * Fused routing metadata, no host synchronisation:
+ *   count64[e]  (optional, int64[E])   rows per expert, overwritten
+ *   seg_off     (int32[E+1])           exclusive prefix, seg_off[E] = N_valid
+ *   pos         (int64[numel])         first N_valid entries written
+ *   inv         (optional, int32[numel])
+ * Stands in for fmoe.functions.count_by_gate + prepare_forward
+ * (fmoe/functions.py:28-75) without their five device-to-host copies.
+ */
+int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
+               int64_t* count64, int32_t* seg_off, int64_t* pos, int32_t* inv,
+               void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ----------------------------------------------------------------- capacity */
+
+/*
+ * eca[w*E+e] = share of expert e's capacity granted to worker w, workers
+ * served in ascending w: grant = proposal if remaining >= proposal, remaining
+ * if remaining >= 0, else 0; remaining -= proposal (the full proposal, also
+ * when clipped).  cap[e] is left holding `remaining`, as the reference's
+ * atomicSub leaves it.  Proposals are truncated to int32 as in the reference.
+ * Replaces fmoe_cuda.limit_by_capacity: cuda/fmoe_cuda.cpp:63-65,
+ * cuda/balancing.cu:9-22, kernel cuda/balancing.cuh:5-30.
+ */
+int fmoe_limit_by_capacity(const int64_t* ec, int32_t* cap, int64_t* eca,
+                           int64_t n_expert, int64_t n_worker, void* stream);
+
+/*
+ * new_gate_idx[i] = gate_idx[i] if fewer than ec[gate_idx[i]] earlier slots
+ * (ascending i) chose the same expert, else -1.  Entries outside [0, E*W)
+ * (including -1) are copied through.  ec[e] is left at ec[e] - count[e], the
+ * state the reference's atomicSub leaves behind.
+ * Replaces fmoe_cuda.prune_gate_by_capacity: cuda/fmoe_cuda.cpp:66-68,
+ * cuda/balancing.cu:24-39, kernel cuda/balancing.cuh:32-56.
+ */
+int fmoe_prune_gate_by_capacity(const int64_t* gate_idx, int64_t* new_gate_idx,
+                                int32_t* ec, int64_t numel, int64_t n_expert,
+                                int64_t n_worker, void* workspace,
+                                int64_t workspace_bytes, void* stream);
+
+/* ----------------------------------------------------------------- dispatch */
+
+/*
+ * out[r] = inp[idx[r] / idx_div] for r < n_rows (rows of `d` elements).
+ * If n_rows_dev is not NULL it points at a device int32 holding the live row
+ * count (<= n_rows) and rows beyond it are left untouched.
+ * Replaces fmoe.functions._local_scatter (fmoe/functions.py:78-80) and the
+ * `pos // top_k` that precedes it (fmoe/layers.py:49-53).
+ */
+int fmoe_local_scatter(const void* inp, const int64_t* idx, void* out,
+                       int64_t n_rows, int64_t d, int64_t idx_div,
+                       const int32_t* n_rows_dev, int dtype, void* stream);
+
+/*
+ * overlap == 0: out = 0 [out_rows, d]; out[pos[r]] = inp[r]  (pos distinct).
+ * overlap != 0: out[p] = sum over {r : pos[r] == p} inp[r]; f32/f64 only
+ *               (device float atomics, summation order unspecified, as with
+ *               the reference's index_add_).
+ * Replaces fmoe.functions._local_gather (fmoe/functions.py:83-90).
+ */
+int fmoe_local_gather(const void* inp, const int64_t* pos, void* out,
+                      int64_t n_rows, int64_t out_rows, int64_t d,
+                      const int32_t* n_rows_dev, int overlap, int dtype,
+                      void* stream);
+
+/*
+ * Gather fused with the top-k weighted combine:
+ *   y[t] = sum_j score[t*k+j] * buf[inv[t*k+j]]   (dropped slots add 0)
+ * fp32 accumulation (fp64 for FMOE_F64), one rounding.
+ * Replaces MOEGather.forward + torch.bmm (fmoe/functions.py:150-176,
+ * fmoe/layers.py:281-295).
+ */
+int fmoe_gather_combine_fwd(const void* buf, const int32_t* inv,
+                            const void* score, void* y, int64_t n_tokens,
+                            int64_t top_k, int64_t d, int dtype, void* stream);
+
+/*
+ * Backward of fmoe_gather_combine_fwd, written straight into expert order:
+ *   dbuf[inv[i]] = score[i] * dy[i / k]          (live slots)
+ *   dscore[i]    = <dy[i / k], buf[inv[i]]>      (0 for dropped slots)
+ * Replaces the bmm backward + MOEGather.backward (fmoe/functions.py:178-193).
+ */
+int fmoe_gather_combine_bwd(const void* dy, const void* buf, const int32_t* inv,
+                            const void* score, void* dbuf, void* dscore,
+                            int64_t n_tokens, int64_t top_k, int64_t d,
+                            int dtype, void* stream);
+
+/*
+ * Backward of the scatter: dx[t] = sum_j dbuf[inv[t*k+j]] over live slots, in
+ * ascending j with fp32 accumulation (deterministic; no float atomics).
+ * Replaces MOEScatter.backward (fmoe/functions.py:126-142).
+ */
+int fmoe_scatter_reduce(const void* dbuf, const int32_t* inv, void* dx,
+                        int64_t n_tokens, int64_t top_k, int64_t d, int dtype,
+                        void* stream);
+
+/* ------------------------------------------------------------ expert GEMMs */
+
+/*
+ * Y[seg_e] = X[seg_e] * W_e^T (+ b_e) for every expert in one launch.
+ *   x [n_rows, in_feat], w [E, out_feat, in_feat], bias [E, out_feat] or NULL,
+ *   y [n_rows, out_feat]; seg_off is a DEVICE int32[E+1].
+ * Rows at or beyond seg_off[E] are not written.  Empty experts cost nothing.
+ * bf16/f16: MFMA with fp32 accumulation.  f32/f64: native accumulation.
+ * Replaces fmoe_cuda.linear_forward: cuda/fmoe_cuda.cpp:48-53,
+ * cuda/parallel_linear.cu:5-50, cuda/parallel_linear.cuh:55-89.
+ */
+int fmoe_grouped_linear_fwd(const void* x, const void* w, const void* bias,
+                            const int32_t* seg_off, void* y, int64_t n_rows,
+                            int64_t in_feat, int64_t out_feat,
+                            int64_t n_expert, int dtype, void* stream);
+
+/*
+ * dX[seg_e] = dY[seg_e] * W_e;  dW_e = dY[seg_e]^T * X[seg_e];
+ * db_e = column sums of dY[seg_e] (only if dbias != NULL).
+ * Experts without rows get dW_e = 0 and db_e = 0.  Any of dx, dw, dbias may
+ * be NULL to skip that product.
+ * Replaces fmoe_cuda.linear_backward: cuda/fmoe_cuda.cpp:54-60,
+ * cuda/parallel_linear.cu:53-96, cuda/parallel_linear.cuh:91-163 and the
+ * column_reduce kernel cuda/parallel_linear.cuh:8-53.
+ */
+int fmoe_grouped_linear_bwd(const void* dy, const void* x, const void* w,
+                            const int32_t* seg_off, void* dx, void* dw,
+                            void* dbias, int64_t n_rows, int64_t in_feat,
+                            int64_t out_feat, int64_t n_expert, int dtype,
+                            void* stream);
+
+/*
+ * seg_off (device int32[E+1]) from HOST int64 counts, the form in which the
+ * reference passes counts to its linear ops (cuda/parallel_linear.cuh:69-70
+ * dereferences expert_count on the host).  `seg_off` must stay alive until
+ * the stream reaches the copy.
+ */
+int fmoe_seg_off_from_host_counts(const int64_t* expert_count_host,
+                                  int64_t n_expert, int32_t* seg_off,
+                                  void* stream);
+
+/*
+ * Selects the grouped-GEMM kernel family for bf16/f16: 0 = automatic (MFMA
+ * where the shape allows), 1 = force the scalar kernel (testing aid).
+ */
+int fmoe_set_gemm_path(int path);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FMOE_HIP_H_ */
