@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the single-GPU MoE-MLP hot path on one MI355X.
+
+A step is one forward + backward pass of the MoE MLP (route, scatter, two
+grouped expert GEMMs with GELU between them, gather fused with the top-k
+combine, and the whole backward) over one batch of synthetic input that is
+already resident in HBM.  Prints ONE JSON line:
+
+  metric / value      MoE-MLP fwd+bwd tokens/s (whole job, one GPU)
+  roofline            the kernel that takes the most time in a step: achieved
+                      algorithmic FLOP/s (or bytes/s) per launch, from HIP
+                      events recorded around every launch inside the timed
+                      region on the stream the kernels run on
+  cpu_baseline        the CPU checker's brute-force layer (torch fp32 on the
+                      host cores) timed on a bounded sample of the same workload
+  kernels             per-kernel average time and achieved rate
+
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+import torch.nn.functional as F  # noqa: E402
+
+# T tokens, d d_model, h d_hidden, E experts, k top-k
+CONFIGS = {
+    "cfg1": dict(T=512, d=128, h=256, E=4, k=2, dtype="f32", x_std=0.02,
+                 note="CPU-plumbing case: N(0,0.02) inputs and weights"),
+    "cfg2": dict(T=8192, d=1024, h=4096, E=16, k=2, dtype="bf16",
+                 note="balanced: gate logits N(0,1)"),
+    "cfg3": dict(T=16384, d=2048, h=8192, E=64, k=2, dtype="bf16", zipf=1.2,
+                 cap_factor=1.25, note="Zipf(1.2) routing, capacity factor 1.25"),
+    "cfg4": dict(T=16384, d=4096, h=14336, E=8, k=2, dtype="bf16",
+                 note="Mixtral-sized layer"),
+    "cfg5": dict(T=8192, d=2048, h=1408, E=128, k=8, dtype="bf16", n_empty=13,
+                 note="fine-grained experts, 13 of 128 empty"),
+}
+DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+PEAK = {"hbm": 8.0e12, "bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
+
+
+def make_routing(cfg: dict, seed: int = 0):
+    """(logits [T, E] float32 or None, idx [T, k] int64 or None): the seeded
+    synthetic routing of a configuration, generated on the CPU."""
+    g = torch.Generator().manual_seed(seed)
+    T, E, k = cfg["T"], cfg["E"], cfg["k"]
+    if "zipf" in cfg:
+        p = torch.arange(1, E + 1, dtype=torch.float64) ** (-cfg["zipf"])
+        idx = torch.multinomial((p / p.sum()).expand(T, -1), k, replacement=False,
+                                generator=g)
+        logits = torch.randn(T, k, generator=g)   # softmax of these gives the scores
+        return logits, idx
+    logits = torch.randn(T, E, generator=g)
+    for e in range(cfg.get("n_empty", 0)):
+        logits[:, (e * E) // cfg["n_empty"]] = float("-inf")
+    return logits, None
+
+
+class PresetGate(torch.nn.Module):
+    """Gate whose decisions are part of the workload, independent of x: top-k of
+    preset logits and the softmax of the k values (the NaiveGate arithmetic,
+    fmoe/gates/naive_gate.py:31-38), or preset Zipf choices clipped to the
+    capacity by the native limit/prune ops."""
+
+    cfg = None  # set before the layer is constructed
+
+    def __init__(self, d_model, num_expert, world_size, top_k=2):
+        super().__init__()
+        cfg = PresetGate.cfg
+        self.top_k = top_k
+        self.num_expert = num_expert
+        logits, idx = make_routing(cfg)
+        self.logits = torch.nn.Parameter(logits)
+        self.register_buffer("idx", idx if idx is not None else torch.zeros(0, dtype=torch.int64))
+        self.capacity = None
+        if "cap_factor" in cfg:
+            self.capacity = math.ceil(cfg["cap_factor"] * cfg["T"] * cfg["k"] / cfg["E"])
+        self.dtype = DTYPES[cfg["dtype"]]
+
+    def forward(self, inp):
+        if self.idx.numel():
+            from fastmoe_amd.gates import limit_by_capacity
+
+            idx = self.idx
+            score = F.softmax(self.logits, dim=-1)
+            if self.capacity is not None:
+                _l, _g, idx = limit_by_capacity(idx, self.num_expert, 1, self.capacity)
+        else:
+            val, idx = torch.topk(self.logits, k=self.top_k, dim=-1, sorted=False)
+            score = F.softmax(val, dim=-1)
+        return idx, score.to(self.dtype)
+
+
+def build_layer(cfg: dict, device="cuda"):
+    from fastmoe_amd import FMoETransformerMLP
+
+    dtype = DTYPES[cfg["dtype"]]
+    PresetGate.cfg = cfg
+    torch.manual_seed(0)
+    layer = FMoETransformerMLP(num_expert=cfg["E"], d_model=cfg["d"], d_hidden=cfg["h"],
+                               top_k=cfg["k"], gate=PresetGate)
+    g = torch.Generator().manual_seed(1)
+    with torch.no_grad():
+        for p in layer.experts.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * 0.02)
+    gate_logits = layer.gate.logits.data
+    layer = layer.to(dtype)
+    layer.gate.logits.data = gate_logits          # routing logits stay fp32
+    layer = layer.to(device)
+    x = (torch.randn(cfg["T"], cfg["d"], generator=g) * cfg.get("x_std", 1.0)).to(dtype)
+    dy = torch.randn(cfg["T"], cfg["d"], generator=g).to(dtype)
+    return layer, x.to(device), dy.to(device)
+
+
+def step(layer, x, dy):
+    for p in layer.parameters():
+        p.grad = None
+    x.grad = None
+    out = layer(x)
+    out.backward(dy)
+    return out
+
+
+# ---------------------------------------------------------------- accounting
+def kernel_work(cfg: dict, n_valid: int):
+    """Algorithmic FLOPs / bytes of ONE launch of each op on this workload."""
+    T, d, h, E, k = cfg["T"], cfg["d"], cfg["h"], cfg["E"], cfg["k"]
+    s = 4 if cfg["dtype"] == "f32" else 2
+    N = T * k
+    gemm = 2.0 * n_valid * d * h
+    return {
+        "grouped_linear_fwd": ("flop", gemm),
+        "grouped_linear_dgrad": ("flop", gemm),
+        "grouped_linear_wgrad": ("flop", gemm),
+        # both layers' bias gradients average to (rows*(d+h)/2) elements read
+        "grouped_linear_bias_grad": ("byte", n_valid * (d + h) / 2.0 * s),
+        "route": ("byte", 8.0 * N + 8.0 * n_valid + 4.0 * N + 8.0 * N),
+        "local_scatter": ("byte", 2.0 * n_valid * d * s + 8.0 * n_valid),
+        "gather_combine_fwd": ("byte", n_valid * d * s + T * d * s + N * (4 + s)),
+        "gather_combine_bwd": ("byte", T * d * s + 2.0 * n_valid * d * s + N * (4 + 2 * s)),
+        "scatter_reduce": ("byte", n_valid * d * s + T * d * s + 4.0 * N),
+        "expert_count": ("byte", 8.0 * N),
+        "limit_by_capacity": ("byte", 20.0 * E),
+        "prune_gate_by_capacity": ("byte", 24.0 * N),
+    }
+
+
+def cpu_baseline(cfg: dict, layer, x, target_seconds: float = 15.0):
+    """The CPU checker's brute-force layer (fp32, all host threads) on the first
+    S tokens of the workload, S sized for about `target_seconds` of work."""
+    from oracle import moe_oracle as O
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    ex = layer.experts
+    with torch.no_grad():
+        idx_all, score_all = layer.gate(x)
+    w = [p.detach().float().cpu() for p in (ex.htoh4.weight, ex.htoh4.bias,
+                                            ex.h4toh.weight, ex.h4toh.bias)]
+
+    def run(S):
+        xs = x[:S].float().cpu().requires_grad_(True)
+        ps = [t.clone().requires_grad_(True) for t in w]
+        t0 = time.perf_counter()
+        out = O.brute_force_moe_mlp(xs, idx_all[:S].cpu(), score_all[:S].float().cpu(), *ps)
+        out.sum().backward()
+        return time.perf_counter() - t0
+
+    T = cfg["T"]
+    probe = max(64, T // 32)
+    run(probe)                                   # warm-up (thread pool, allocator)
+    t_probe = run(probe)
+    S = int(min(T, max(probe, probe * target_seconds / 3.0 / max(t_probe, 1e-6))))
+    times = [run(S) for _ in range(3)]
+    best = min(times)
+    return {
+        "value": S / best,
+        "unit": "tokens/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"first {S} of {T} tokens of {cfg['name']}, fp32 torch on the host, "
+                  f"fwd+bwd, best of 3 ({best:.3f} s)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="cfg2", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures ONE GPU: this build has no multi-GPU path "
+                 "(world_size is 1); run with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (there is no CPU fallback of the hot path)")
+
+    from fastmoe_amd import fmoe_cuda
+
+    cfg = dict(CONFIGS[args.config], name=args.config)
+    layer, x, dy = build_layer(cfg)
+    x.requires_grad_(True)
+
+    for _ in range(args.warmup):
+        step(layer, x, dy)
+    torch.cuda.synchronize()
+
+    records = []
+    fmoe_cuda.profile_hook = lambda name, a, b: records.append((name, a, b))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(layer, x, dy)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    fmoe_cuda.profile_hook = None
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    with torch.no_grad():
+        idx, _ = layer.gate(x)
+    n_valid = int((idx >= 0).sum().item())
+
+    work = kernel_work(cfg, n_valid)
+    per = {}
+    for name, a, b in records:
+        per.setdefault(name, []).append(a.elapsed_time(b))
+    kernels = {}
+    for name, ts in per.items():
+        avg_ms = sum(ts) / len(ts)
+        kind, amount = work.get(name, ("byte", 0.0))
+        rate = amount / (avg_ms * 1e-3) if avg_ms > 0 else 0.0
+        peak = PEAK[cfg["dtype"]] if kind == "flop" else PEAK["hbm"]
+        kernels[name] = {
+            "launches_per_step": len(ts) / args.steps,
+            "avg_us": round(avg_ms * 1e3, 2),
+            "total_ms_per_step": round(sum(ts) / args.steps, 4),
+            ("tflops" if kind == "flop" else "gbps"):
+                round(rate / (1e12 if kind == "flop" else 1e9), 2),
+            "frac_of_peak": round(rate / peak, 4),
+        }
+    dom = max(kernels, key=lambda n: kernels[n]["total_ms_per_step"])
+    kind, amount = work[dom]
+    avg_s = kernels[dom]["avg_us"] * 1e-6
+    if kind == "flop":
+        roofline = {"kernel": dom, "bound": "mfma", "achieved": round(amount / avg_s / 1e12, 2),
+                    "peak": PEAK[cfg["dtype"]] / 1e12, "unit": "TFLOP/s"}
+    else:
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": round(amount / avg_s / 1e9, 2),
+                    "peak": PEAK["hbm"] / 1e9, "unit": "GB/s"}
+    roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+    roofline["traffic"] = None
+    roofline["avg_launch_us"] = kernels[dom]["avg_us"]
+
+    result = {
+        "metric": "MoE-MLP fwd+bwd tokens/s @1 MI355X",
+        "value": round(cfg["T"] / (ms_per_step * 1e-3), 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {
+            "workload": (f"{args.config}: {cfg['T']} tokens, d_model {cfg['d']}, d_hidden "
+                         f"{cfg['h']}, {cfg['E']} experts, top-{cfg['k']}, {cfg['dtype']}; "
+                         f"{cfg['note']}"),
+            "routed_slots": cfg["T"] * cfg["k"],
+            "live_slots": n_valid,
+            "gemm_flops_per_step": 12.0 * n_valid * cfg["d"] * cfg["h"],
+        },
+        "gemm_tflops_overall": round(12.0 * n_valid * cfg["d"] * cfg["h"]
+                                     / (ms_per_step * 1e-3) / 1e12, 2),
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(cfg, layer, x.detach())
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

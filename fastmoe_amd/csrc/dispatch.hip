@@ -109,6 +109,21 @@ __global__ __launch_bounds__(kDispThreads) void add_rows_kernel(
   }
 }
 
+// Value held by lane j (wave-uniform j), readable also when lane j itself is
+// masked off in the current branch: v_readlane ignores EXEC.
+__device__ __forceinline__ int32_t lane_value(int32_t v, int j) {
+  return __builtin_amdgcn_readlane(v, j);
+}
+__device__ __forceinline__ float lane_value(float v, int j) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), j));
+}
+__device__ __forceinline__ double lane_value(double v, int j) {
+  const long long b = __double_as_longlong(v);
+  const int lo = __builtin_amdgcn_readlane((int)(b & 0xffffffffLL), j);
+  const int hi = __builtin_amdgcn_readlane((int)(b >> 32), j);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
 // ------------------------------------------------ gather fused with combine
 // y[t] = sum_j score[t,j] * buf[inv[t,j]]; score == nullptr means weight 1
 // (the scatter backward).  VEC elements per lane per step (16 bytes, or 1).
@@ -136,8 +151,10 @@ __global__ __launch_bounds__(kDispThreads) void combine_fwd_kernel(
 #pragma unroll
       for (int v = 0; v < VEC; ++v) acc[v] = 0;
       for (int j = 0; j < top_k; ++j) {
-        const int32_t r = __shfl(my_r, j, kWave);
-        const acc_t s = __shfl(my_s, j, kWave);
+        // lanes beyond the row's last pack are not in this loop, so a
+        // shuffle could not read them; lane_value can
+        const int32_t r = lane_value(my_r, j);
+        const acc_t s = lane_value(my_s, j);
         if (r < 0) continue;
         const Pk p = *reinterpret_cast<const Pk*>(buf + (int64_t)r * d + c * VEC);
 #pragma unroll
@@ -172,8 +189,8 @@ __global__ __launch_bounds__(kDispThreads) void combine_bwd_kernel(
       my_s = Elem<T>::to_acc(score[t * top_k + lane]);
     }
     for (int j = 0; j < top_k; ++j) {
-      const int32_t r = __shfl(my_r, j, kWave);
-      const acc_t s = __shfl(my_s, j, kWave);
+      const int32_t r = lane_value(my_r, j);
+      const acc_t s = lane_value(my_s, j);
       acc_t dot = 0;
       if (r >= 0) {
         for (int64_t c = lane; c < row_vecs; c += kWave) {

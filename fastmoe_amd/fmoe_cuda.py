@@ -72,6 +72,35 @@ class _on:
             self.guard.__exit__(*exc)
 
 
+# Optional per-op timing: when `profile_hook` is set to a callable it receives
+# (op name, start event, end event) for every launch group, with both events
+# recorded on the stream the kernels run on.  Off (None) by default.
+profile_hook = None
+
+
+class _launch(_on):
+    """Device guard plus, when profiling, an event pair around the launches."""
+
+    def __init__(self, t: torch.Tensor, name: str):
+        super().__init__(t)
+        self.name = name
+        self.t = t
+        self.ev = None
+
+    def __enter__(self):
+        super().__enter__()
+        if profile_hook is not None:
+            self.ev = (torch.cuda.Event(enable_timing=True),
+                       torch.cuda.Event(enable_timing=True))
+            self.ev[0].record(torch.cuda.current_stream(self.t.device))
+
+    def __exit__(self, *exc):
+        if self.ev is not None:
+            self.ev[1].record(torch.cuda.current_stream(self.t.device))
+            profile_hook(self.name, self.ev[0], self.ev[1])
+        super().__exit__(*exc)
+
+
 def _workspace(numel: int, n_expert: int, device) -> torch.Tensor:
     nbytes = _L.fmoe_route_workspace_bytes(numel, n_expert)
     _need(nbytes >= 0, "route workspace: bad sizes")
@@ -87,7 +116,7 @@ def expert_count(gate_idx: torch.Tensor, expert_count: torch.Tensor) -> None:
     cuda/local_exchange.cu:22-32."""
     _dev(gate_idx, "gate_idx", torch.int64)
     _dev(expert_count, "expert_count", torch.int32)
-    with _on(gate_idx):
+    with _launch(gate_idx, "expert_count"):
         _lib.check(
             _L.fmoe_expert_count(gate_idx.data_ptr(), gate_idx.numel(),
                                  expert_count.data_ptr(), expert_count.numel(),
@@ -103,7 +132,7 @@ def assign_pos(cum_count: torch.Tensor, gate: torch.Tensor, pos: torch.Tensor) -
     _dev(pos, "pos", torch.int64)
     n, e = gate.numel(), cum_count.numel()
     ws = _workspace(n, e, gate.device)
-    with _on(gate):
+    with _launch(gate, "assign_pos"):
         _lib.check(
             _L.fmoe_assign_pos(cum_count.data_ptr(), gate.data_ptr(), pos.data_ptr(),
                                n, e, ws.data_ptr(), ws.numel(), _stream(gate)),
@@ -166,7 +195,7 @@ def limit_by_capacity(expert_count: torch.Tensor, capacity: torch.Tensor,
     _need(expert_count.numel() >= n_expert * n_worker, "expert_count too short")
     _need(capacity.numel() >= n_expert, "capacity too short")
     ack = torch.empty_like(expert_count)
-    with _on(expert_count):
+    with _launch(expert_count, "limit_by_capacity"):
         _lib.check(
             _L.fmoe_limit_by_capacity(expert_count.data_ptr(), capacity.data_ptr(),
                                       ack.data_ptr(), n_expert, n_worker,
@@ -185,7 +214,7 @@ def prune_gate_by_capacity(gate_idx: torch.Tensor, expert_count: torch.Tensor,
     new_gate = torch.empty_like(gate_idx)
     n = gate_idx.numel()
     ws = _workspace(n, n_expert * n_worker, gate_idx.device)
-    with _on(gate_idx):
+    with _launch(gate_idx, "prune_gate_by_capacity"):
         _lib.check(
             _L.fmoe_prune_gate_by_capacity(gate_idx.data_ptr(), new_gate.data_ptr(),
                                            expert_count.data_ptr(), n, n_expert,
@@ -208,7 +237,7 @@ def local_scatter(inp: torch.Tensor, pos: torch.Tensor, idx_div: int = 1,
     dt = _dt(inp, "inp")
     n, d = pos.numel(), inp.shape[1]
     out = torch.empty((n, d), dtype=inp.dtype, device=inp.device)
-    with _on(inp):
+    with _launch(inp, "local_scatter"):
         _lib.check(
             _L.fmoe_local_scatter(inp.data_ptr(), pos.data_ptr(), out.data_ptr(), n, d,
                                   idx_div, _ptr(n_rows_dev), dt, _stream(inp)),
@@ -232,7 +261,7 @@ def local_gather(inp: torch.Tensor, pos: torch.Tensor, out_batch_size: int,
         # half types accumulate in fp32, rounded once at the end
         acc = local_gather(inp.float(), pos, out_batch_size, True, n_rows_dev)
         return acc.to(inp.dtype)
-    with _on(inp):
+    with _launch(inp, "local_gather"):
         _lib.check(
             _L.fmoe_local_gather(inp.data_ptr(), pos.data_ptr(), out.data_ptr(), n,
                                  out_batch_size, d, _ptr(n_rows_dev),
@@ -258,7 +287,7 @@ def route(gate: torch.Tensor, n_expert: int, want_inv: bool = True
     pos = torch.empty(n, dtype=torch.int64, device=dev)
     inv = torch.empty(n, dtype=torch.int32, device=dev) if want_inv else None
     ws = _workspace(n, n_expert, dev)
-    with _on(gate):
+    with _launch(gate, "route"):
         _lib.check(
             _L.fmoe_route(gate.data_ptr(), n, n_expert, count.data_ptr(),
                           seg.data_ptr(), pos.data_ptr(), _ptr(inv), ws.data_ptr(),
@@ -282,7 +311,7 @@ def grouped_linear_fwd(x: torch.Tensor, seg_off: torch.Tensor, weight: torch.Ten
         _need(tuple(bias.shape) == (e, out_f), "bias must be [E, out]")
     dt = _dt(x, "x")
     y = torch.empty((x.shape[0], out_f), dtype=x.dtype, device=x.device)
-    with _on(x):
+    with _launch(x, "grouped_linear_fwd"):
         _lib.check(
             _L.fmoe_grouped_linear_fwd(x.data_ptr(), weight.data_ptr(), _ptr(bias),
                                        seg_off.data_ptr(), y.data_ptr(), x.shape[0],
@@ -308,12 +337,19 @@ def grouped_linear_bwd(dy: torch.Tensor, x: torch.Tensor, seg_off: torch.Tensor,
     dx = torch.empty((n, in_f), dtype=dy.dtype, device=dy.device) if need_dx else None
     dw = torch.empty_like(weight) if need_dw else None
     db = torch.empty((e, out_f), dtype=dy.dtype, device=dy.device) if need_bias else None
-    with _on(dy):
-        _lib.check(
-            _L.fmoe_grouped_linear_bwd(dy.data_ptr(), x.data_ptr(), weight.data_ptr(),
-                                       seg_off.data_ptr(), _ptr(dx), _ptr(dw), _ptr(db),
-                                       n, in_f, out_f, e, dt, _stream(dy)),
-            "grouped_linear_bwd")
+    # one C call per product, so a profile hook sees each kernel on its own
+    for name, a, b, c in (("grouped_linear_dgrad", dx, None, None),
+                          ("grouped_linear_wgrad", None, dw, None),
+                          ("grouped_linear_bias_grad", None, None, db)):
+        if a is None and b is None and c is None:
+            continue
+        with _launch(dy, name):
+            _lib.check(
+                _L.fmoe_grouped_linear_bwd(dy.data_ptr(), x.data_ptr(),
+                                           weight.data_ptr(), seg_off.data_ptr(),
+                                           _ptr(a), _ptr(b), _ptr(c), n, in_f, out_f,
+                                           e, dt, _stream(dy)),
+                name)
     return dx, dw, db
 
 
@@ -327,7 +363,7 @@ def gather_combine_fwd(buf: torch.Tensor, inv: torch.Tensor, score: torch.Tensor
           "inv/score must have n_tokens*top_k entries")
     d = buf.shape[1]
     y = torch.empty((n_tokens, d), dtype=buf.dtype, device=buf.device)
-    with _on(buf):
+    with _launch(buf, "gather_combine_fwd"):
         _lib.check(
             _L.fmoe_gather_combine_fwd(buf.data_ptr(), inv.data_ptr(), score.data_ptr(),
                                        y.data_ptr(), n_tokens, top_k, d,
@@ -348,7 +384,7 @@ def gather_combine_bwd(dy: torch.Tensor, buf: torch.Tensor, inv: torch.Tensor,
     _need(tuple(dy.shape) == (n_tokens, d), "dy must be [n_tokens, d]")
     dbuf = torch.empty_like(buf)
     dscore = torch.empty((n_tokens, top_k), dtype=dy.dtype, device=dy.device)
-    with _on(dy):
+    with _launch(dy, "gather_combine_bwd"):
         _lib.check(
             _L.fmoe_gather_combine_bwd(dy.data_ptr(), buf.data_ptr(), inv.data_ptr(),
                                        score.data_ptr(), dbuf.data_ptr(),
@@ -366,7 +402,7 @@ def scatter_reduce(dbuf: torch.Tensor, inv: torch.Tensor, n_tokens: int,
     _need(inv.numel() == n_tokens * top_k, "inv must have n_tokens*top_k entries")
     d = dbuf.shape[1]
     dx = torch.empty((n_tokens, d), dtype=dbuf.dtype, device=dbuf.device)
-    with _on(dbuf):
+    with _launch(dbuf, "scatter_reduce"):
         _lib.check(
             _L.fmoe_scatter_reduce(dbuf.data_ptr(), inv.data_ptr(), dx.data_ptr(),
                                    n_tokens, top_k, d, _dt(dbuf, "dbuf"),
