@@ -28,6 +28,7 @@ FLAGS = [
     "-fPIC",
     "-Wall",
     "-Wno-unused-function",
+    "-Wno-inline-asm",   # m0 is written by the LDS-copy instruction sequence
     # keep the compiler from forming packed-fp32 instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]

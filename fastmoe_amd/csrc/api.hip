@@ -2,6 +2,7 @@
 // bias gradient) and the host-count upload.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include "gemm.h"
 
@@ -9,6 +10,8 @@ namespace fmoe {
 
 static thread_local char g_err[512] = "";
 static int g_gemm_path = 0;  // 0 = automatic, 1 = scalar kernel only
+// tuning aid: FMOE_GEMM_TILE=1..3 forces one MFMA tile shape (0 / unset = automatic)
+static int g_tile = getenv("FMOE_GEMM_TILE") ? atoi(getenv("FMOE_GEMM_TILE")) : 0;
 
 int set_error(int code, const char* fmt, ...) {
   va_list ap;
@@ -156,7 +159,7 @@ extern "C" int fmoe_grouped_linear_fwd(const void* x, const void* w,
   if (n_rows == 0) return FMOE_OK;
   FMOE_REQUIRE(x && w && seg_off && y, FMOE_ERR_INVALID,
                "grouped_linear_fwd: null pointer");
-  GemmArgs g{x, w, y, bias, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert};
+  GemmArgs g{x, w, y, bias, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
   return run_gemm(GEMM_FWD, g, dtype, (hipStream_t)stream);
 }
 
@@ -175,7 +178,7 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
   hipStream_t s = (hipStream_t)stream;
   if (dx && n_rows > 0) {
     FMOE_REQUIRE(w != nullptr, FMOE_ERR_INVALID, "grouped_linear_bwd: w is null");
-    GemmArgs g{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert};
+    GemmArgs g{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
     rc = run_gemm(GEMM_DGRAD, g, dtype, s);
     if (rc) return rc;
   }
@@ -183,7 +186,7 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
     // runs also for n_rows == 0: experts without rows get zero gradients
     FMOE_REQUIRE(n_rows == 0 || x != nullptr, FMOE_ERR_INVALID,
                  "grouped_linear_bwd: x is null");
-    GemmArgs g{dy, x, dw, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert};
+    GemmArgs g{dy, x, dw, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
     rc = run_gemm(GEMM_WGRAD, g, dtype, s);
     if (rc) return rc;
   }

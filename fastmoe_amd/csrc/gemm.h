@@ -21,6 +21,7 @@ struct GemmArgs {
   int in_feat;
   int out_feat;
   int n_expert;
+  int tile;             // 0 = choose the tile shape automatically, 1..3 = force one
 };
 
 // Virtual row-tile index space for the ragged products: expert e owns the

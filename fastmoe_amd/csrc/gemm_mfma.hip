@@ -5,15 +5,26 @@
 //
 // Block tile BM x BN x BK with WM x WN wave64s; every wave owns a
 // (BM/WM) x (BN/WN) patch as a grid of 32x32 accumulators fed by
-// v_mfma_f32_32x32x16_{bf16,f16}.  Operand tiles go global -> registers -> LDS
-// (double buffered) as 16-byte packs:
-//   * an operand whose K index is contiguous in memory is stored [row][BK]
-//     with the 16-byte pack index XOR-swizzled by the row, and a lane reads
-//     its 8 consecutive K values with one ds_read_b128;
-//   * an operand whose K index is the strided one (W in DGRAD, both operands
-//     in WGRAD) is stored as it arrives, [k][row], and read back transposed.
-// Loads are predicated per 16-byte pack and zero-filled, so partial tiles in
-// M, N and K need no separate kernel.
+// v_mfma_f32_32x32x16_{bf16,f16}.
+//
+// Operand tiles go from HBM/L2 straight into LDS with buffer_load_dwordx4 ...
+// lds (no staging registers): one wave instruction fills 1 KiB of LDS, lane l
+// writing bytes [16 l, 16 l + 16).  Which 16-byte pack of the tile a lane
+// fetches is chosen so that the pack lands where the bank-conflict-free read
+// pattern expects it:
+//   * K contiguous in memory (X, dY as the A operand, W in FWD): LDS is
+//     [row][BK]; pack index XOR ((row ^ row/8) & 7); a lane reads its 8
+//     consecutive K values with one ds_read_b128.
+//   * K strided in memory (W in DGRAD, both operands in WGRAD): LDS is
+//     [k][rows] as it arrives; 32-byte segment index XOR (k & 3); fragments
+//     come back through ds_read_b64_tr_b16, which transposes 16-bit elements
+//     across groups of 16 lanes.
+// Out-of-range packs (ragged M, N or K edges) are pointed beyond the buffer
+// descriptor's num_records and arrive as zeros, so there are no edge kernels
+// and no branches in the load path.
+//
+// Two LDS stages: the loads of K-slice t+1 are in flight while slice t feeds
+// the MFMAs; one barrier per slice.
 //
 // Operand roles follow cuda/parallel_linear.cuh:69-87,124-147 of the
 // reference; the per-expert cuBLAS loop there becomes a tile index space.
@@ -24,6 +35,9 @@ namespace fmoe {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 template <typename T> struct Mma;
 template <> struct Mma<__hip_bfloat16> {
@@ -39,104 +53,182 @@ template <> struct Mma<__half> {
   }
 };
 
-constexpr int kTrPad = 8;  // elements of padding per [k] row of a transposed tile
+constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any num_records used here
+constexpr int kRsrcFlags = 0x00020000;         // raw buffer, 32-bit data format
+constexpr int kImmSpan = 3072;                 // largest immediate offset used (3 KiB)
 
-// One operand tile of R rows (the M or N index) by BK: how it is fetched,
-// where it lands in LDS and how a wave reads its MFMA fragment back.
-// KC == true : memory is [row][k] (k contiguous), LDS is [row][BK] swizzled.
-// KC == false: memory is [k][row] (row contiguous), LDS is [k][R + kTrPad].
-template <int R, int BK, int NT, bool KC>
-struct OperandTile {
-  static constexpr int kChunks = R * BK / 8;
-  static constexpr int kPerThread = kChunks / NT;
-  static_assert(kChunks % NT == 0, "tile must split evenly over the threads");
-  static constexpr int kCpr = KC ? BK / 8 : R / 8;  // 16-byte packs per LDS row
-  static constexpr int kLdsElems = KC ? R * BK : BK * (R + kTrPad);
+// One operand tile of R rows (the M or N index) by BK values of K.
+// KC == true : memory is [row][k] (k contiguous), LDS is [row][BK].
+// KC == false: memory is [k][row] (row contiguous), LDS is [k][R].
+//
+// A wave copies kPerWave consecutive 1 KiB blocks of the tile per K-slice, in
+// groups of up to four instructions that share one M0 (LDS base) and step
+// through the blocks with the instruction's immediate offset.  The hardware
+// adds that immediate to the global offset as well, so the descriptor base is
+// set kImmSpan bytes low and every lane offset carries the difference.
+template <int R, int BK, int NW, bool KC>
+struct DmaTile {
+  static constexpr int kBytes = R * BK * 2;
+  static constexpr int kBlocks = kBytes / 1024;     // one wave instruction each
+  static constexpr int kPerWave = kBlocks / NW;
+  static constexpr int kGroup = kPerWave >= 4 ? 4 : kPerWave;
+  static constexpr int kGroups = kPerWave / kGroup;
+  static_assert(kBlocks % NW == 0 && kPerWave % kGroup == 0, "tile must split evenly");
+  static_assert(BK == 64 || BK == 32, "swizzles below assume 128- or 64-byte [row][BK] rows");
+  static constexpr int kRowPacks = R / 8;           // packs per [k] row (KC == false)
+  static constexpr int kKPacks = BK / 8;            // packs per [row] row (KC == true)
 
-  __device__ static __forceinline__ int swz(int row) {
-    return (row ^ (row >> 3)) & (BK / 8 - 1);
+  // XOR applied to the pack index of a [row][BK] row so that 16 consecutive
+  // rows read at the same K offset cover all 64 LDS banks.
+  __device__ static __forceinline__ int row_swizzle(int row) {
+    return BK == 64 ? ((row & 7) ^ ((row >> 3) & 1)) : ((row >> 2) & 3);
   }
 
-  uint4 regs[kPerThread];
+  // per lane
+  uint32_t voff[kPerWave];  // byte offset of this lane's pack (+ immediate compensation)
+  int kpack[kPerWave];      // KC: K offset (elements) of the pack inside the slice
+  // per wave (scalar registers)
+  uint32_t base_lo, base_hi;  // descriptor base of the current slice, kImmSpan low
+  int remaining;              // bytes from the slice origin to the end of the valid data
+  int step;                   // bytes between consecutive slices
+  int k_left;                 // K values from the slice start to the end of K
 
-  // base points at element (row 0, k 0) of the operand for this problem;
-  // ld is the stride of the non-contiguous index; limits are exclusive.
-  __device__ __forceinline__ void fetch(const uint16_t* base, int64_t ld, int r0,
-                                        int k0, int r_limit, int k_limit, int tid) {
+  // origin: element (row 0, k 0) of the tile; ld: elements between rows (KC)
+  // or between consecutive k (not KC); r_valid rows and k_total values of K
+  // exist; r_span = valid elements along the contiguous index of a [k] row.
+  __device__ __forceinline__ void init(const uint16_t* origin, int wave, int lane,
+                                       int ld, int r_valid, int r_span, int k_total) {
 #pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const int q = tid + i * NT;
-      const int major = q / kCpr, minor = (q % kCpr) * 8;
-      uint4 v = make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < kPerWave; ++i) {
+      const int b = wave * kPerWave + i;
+      const uint32_t comp = (uint32_t)(kImmSpan - (i % kGroup) * 1024);
       if (KC) {
-        const int r = r0 + major, k = k0 + minor;
-        if (r < r_limit && k < k_limit)
-          v = *reinterpret_cast<const uint4*>(base + (int64_t)r * ld + k);
+        const int row = b * (64 / kKPacks) + lane / kKPacks;
+        const int kc = (lane % kKPacks) ^ row_swizzle(row);
+        voff[i] = (uint32_t)(row * ld + kc * 8) * 2u + comp;
+        kpack[i] = kc * 8;
       } else {
-        const int k = k0 + major, r = r0 + minor;
-        if (k < k_limit && r < r_limit)
-          v = *reinterpret_cast<const uint4*>(base + (int64_t)k * ld + r);
+        const int k = b * (64 / kRowPacks) + lane / kRowPacks;
+        const int rc = (lane % kRowPacks) ^ ((k & 3) << 1);
+        voff[i] = rc * 8 < r_valid ? (uint32_t)(k * ld + rc * 8) * 2u + comp : kOutOfRange;
+        kpack[i] = 0;
       }
-      regs[i] = v;
     }
+    const uint64_t p = (uint64_t)origin - kImmSpan;
+    base_lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    base_hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32));
+    // everything past the ragged edge is beyond num_records and reads as zero
+    remaining = KC ? ((r_valid - 1) * ld + k_total) * 2
+                   : ((k_total - 1) * ld + r_span) * 2;
+    if (k_total <= 0) remaining = 0;
+    remaining = __builtin_amdgcn_readfirstlane(remaining);
+    step = __builtin_amdgcn_readfirstlane((KC ? BK : BK * ld) * 2);
+    k_left = k_total;
   }
 
-  __device__ __forceinline__ void stash(uint16_t* lds, int tid) const {
+  // Moves on to the next K-slice (a slice past the end of K reads all zeros).
+  __device__ __forceinline__ void advance() {
+    const uint64_t p = (((uint64_t)base_hi << 32) | base_lo) + (uint32_t)step;
+    base_lo = (uint32_t)p;
+    base_hi = (uint32_t)(p >> 32);
+    remaining -= step;
+    k_left -= BK;
+  }
+
+  // Group gi of this wave's copy instructions of the current slice into the
+  // tile at LDS byte address `tile_lds`.
+  //
+  // Written as inline assembly on purpose: the compiler then neither knows
+  // that LDS is being written nor counts the loads in vmcnt, so it does not
+  // put a full vmcnt(0) wait in front of every LDS read of the OTHER stages.
+  // The kernel waits for a slice explicitly and publishes it with a barrier
+  // before anyone reads it.
+  __device__ __forceinline__ void issue_group(int gi, uint32_t tile_lds, int wave) const {
+    i32x4_t rsrc;
+    rsrc[0] = (int)base_lo;
+    rsrc[1] = (int)(base_hi & 0xffffu);                       // stride 0
+    rsrc[2] = remaining > 0 ? remaining + kImmSpan : 0;       // num_records
+    rsrc[3] = kRsrcFlags;
+    uint32_t off[kGroup];
 #pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const int q = tid + i * NT;
-      const int major = q / kCpr, minor = q % kCpr;
-      int off;
-      if (KC) off = major * BK + ((minor ^ swz(major)) * 8);
-      else off = major * (R + kTrPad) + minor * 8;
-      *reinterpret_cast<uint4*>(lds + off) = regs[i];
+    for (int j = 0; j < kGroup; ++j) {
+      off[j] = voff[gi * kGroup + j];
+      if (KC) off[j] = kpack[gi * kGroup + j] < k_left ? off[j] : kOutOfRange;  // K tail
+    }
+    const uint32_t dst = tile_lds + (uint32_t)(wave * kPerWave + gi * kGroup) * 1024u;
+    if constexpr (kGroup == 4) {
+      asm volatile(
+          "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+          "buffer_load_dwordx4 %1, %5, 0 offen lds\n\t"
+          "buffer_load_dwordx4 %2, %5, 0 offen offset:1024 lds\n\t"
+          "buffer_load_dwordx4 %3, %5, 0 offen offset:2048 lds\n\t"
+          "buffer_load_dwordx4 %4, %5, 0 offen offset:3072 lds"
+          :: "s"(dst), "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "s"(rsrc)
+          : "memory", "m0");
+    } else if constexpr (kGroup == 2) {
+      asm volatile(
+          "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+          "buffer_load_dwordx4 %1, %3, 0 offen lds\n\t"
+          "buffer_load_dwordx4 %2, %3, 0 offen offset:1024 lds"
+          :: "s"(dst), "v"(off[0]), "v"(off[1]), "s"(rsrc) : "memory", "m0");
+    } else {
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                   :: "s"(dst), "v"(off[0]), "s"(rsrc) : "memory", "m0");
     }
   }
 
-  // fragment of the 32-row sub-tile starting at `row32` for K step `kk`
-  // (16 values of K): lane l gets row row32 + l%32, K values 8*(l/32) .. +7.
+  // MFMA fragment of the 32-row sub-tile starting at `row32`, K step `kk`
+  // (16 values of K): lane l holds row row32 + l%32, K values 8*(l/32) .. +7.
   __device__ static __forceinline__ uint4 frag(const uint16_t* lds, int row32,
                                                int kk, int lane) {
-    const int r = row32 + (lane & 31);
-    const int half = lane >> 5;
     if (KC) {
-      const int chunk = kk * 2 + half;
-      return *reinterpret_cast<const uint4*>(lds + r * BK + ((chunk ^ swz(r)) * 8));
+      const int r = row32 + (lane & 31);
+      const int pack = (kk * 2 + (lane >> 5)) ^ row_swizzle(r);
+      return *reinterpret_cast<const uint4*>(lds + r * BK + pack * 8);
     } else {
-      const uint16_t* p = lds + (kk * 16 + half * 8) * (R + kTrPad) + r;
-      uint32_t w[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t lo = p[(2 * j) * (R + kTrPad)];
-        const uint32_t hi = p[(2 * j + 1) * (R + kTrPad)];
-        w[j] = lo | (hi << 16);
-      }
-      return make_uint4(w[0], w[1], w[2], w[3]);
+      // ds_read_b64_tr_b16: within 16 lanes, lane i supplies the address of
+      // elements [k + i/4][m + 4*(i%4) .. +3] and receives [k .. k+3][m + i].
+      const int k = kk * 16 + 8 * (lane >> 5) + ((lane & 15) >> 2);
+      const int m = row32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+      const int seg = (m >> 4) ^ (k & 3), within = m & 15;   // 32-byte segments
+      const uint16_t* p = lds + k * R + seg * 16 + within;
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4_t*)(p));
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4_t*)(p + 4 * R));
+      uint4 out;
+      const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+      out.x = l2.x; out.y = l2.y; out.z = h2.x; out.w = h2.y;
+      return out;
     }
   }
 };
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int MODE>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
                                                                 int tiles_n,
                                                                 int tiles_m) {
-  constexpr int NT = WM * WN * 64;
+  constexpr int NW = WM * WN;
+  constexpr int NT = NW * 64;
   constexpr bool A_KC = MODE != GEMM_WGRAD;
   constexpr bool B_KC = MODE == GEMM_FWD;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % 16 == 0, "tile shape");
-  using ATile = OperandTile<BM, BK, NT, A_KC>;
-  using BTile = OperandTile<BN, BK, NT, B_KC>;
+  static_assert(NS >= 4 && NS <= 6, "LDS stages");
+  using ATile = DmaTile<BM, BK, NW, A_KC>;
+  using BTile = DmaTile<BN, BK, NW, B_KC>;
+  constexpr int kStageBytes = ATile::kBytes + BTile::kBytes;
+  constexpr int kStageElems = kStageBytes / 2;
+  constexpr int kLoads = ATile::kPerWave + BTile::kPerWave;  // per wave per slice
+  constexpr int kGroups = ATile::kGroups + BTile::kGroups;   // asm groups per slice
+  static_assert(kLoads * (NS - 3) < 64, "vmcnt is a 6-bit counter");
 
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  // [A buffer 0][A buffer 1][B buffer 0][B buffer 1]
-  uint16_t* const lds_a = smem;
-  uint16_t* const lds_b = smem + 2 * ATile::kLdsElems;
+  extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];  // [stage][A | B]
   __shared__ int s_expert;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave / WN, wave_n = wave % WN;
   const int in_f = g.in_feat, out_f = g.out_feat;
 
@@ -164,11 +256,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   }
   e = __builtin_amdgcn_readfirstlane(e);
   m_tile = __builtin_amdgcn_readfirstlane(m_tile);
-  const int row0 = g.seg_off[e];
-  const int cnt = g.seg_off[e + 1] - row0;
+  const int row0 = __builtin_amdgcn_readfirstlane(g.seg_off[e]);
+  const int cnt = __builtin_amdgcn_readfirstlane(g.seg_off[e + 1]) - row0;
 
-  int M, N, K;
-  int64_t lda, ldb, ldc;
+  int M, N, K, lda, ldb, ldc;
   const uint16_t *A, *B;
   T* C;
   if (MODE == GEMM_FWD) {
@@ -189,7 +280,23 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   }
   const int m0 = m_tile * BM, n0 = n_tile * BN;
   if (m0 >= M || n0 >= N) return;
+  const int m_valid = min(BM, M - m0), n_valid = min(BN, N - n0);
 
+  const uint32_t lds_base = (uint32_t)(size_t)(lds_ptr_t)smem;
+  ATile ta;
+  BTile tb;
+  ta.init(A_KC ? A + (int64_t)m0 * lda : A + m0, wave, lane, lda, m_valid, M - m0, K);
+  tb.init(B_KC ? B + (int64_t)n0 * ldb : B + n0, wave, lane, ldb, n_valid, N - n0, K);
+
+  // gi-th copy group of the current slice (A tile's groups first)
+  auto issue_group = [&](int gi, uint32_t stage_lds) {
+    if (gi < ATile::kGroups) ta.issue_group(gi, stage_lds, wave);
+    else tb.issue_group(gi - ATile::kGroups, stage_lds + ATile::kBytes, wave);
+  };
+
+  // acc[i][j] holds the TRANSPOSE of the 32x32 block (i, j) of C: the MFMA is
+  // fed (B fragment, A fragment), so a lane ends up with 4 consecutive columns
+  // of one row of C per group of 4 accumulators and can store them as 8 bytes.
   f32x16_t acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -198,76 +305,126 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  ATile ta;
-  BTile tb;
+  // ---- software pipeline over the K-slices (NS LDS stages, NS >= 4)
+  //
+  // At the top of iteration kt: slices kt and kt+1 are visible to every wave,
+  // slice kt+2 is in flight, the MFMA fragments of (kt, K step 0) are already
+  // in registers, and the stage of slice kt-1 is free.  The iteration
+  //   * issues the copy of slice kt+NS-1 into that free stage, its groups of
+  //     copy instructions spread between the MFMAs,
+  //   * runs the MFMAs of slice kt, reading the fragments of the next K step
+  //     one LDS read behind each MFMA; the last K step prefetches the first
+  //     fragments of slice kt+1, so the MFMA pipe does not drain at the barrier,
+  //   * waits until its own share of slice kt+2 has landed and meets the other
+  //     waves at the barrier, which publishes slice kt+2 and frees stage kt.
+  // Slices past the end of K are zero-filled dummies; nothing is conditional.
+  constexpr int KK = BK / 16;                    // MFMA K steps per slice
+  constexpr int kMmaPerSlice = KK * TM * TN;
+  constexpr int kEvery = kMmaPerSlice / kGroups; // MFMAs between two copy groups
+  static_assert(KK % 2 == 0, "fragment double buffer is indexed by the parity of the K step");
+  static_assert(kEvery >= 1 && TM + TN <= TM * TN, "interleaving plan");
+
   const int k_tiles = (K + BK - 1) / BK;
-  if (k_tiles > 0) {
-    ta.fetch(A, lda, m0, 0, M, K, tid);
-    tb.fetch(B, ldb, n0, 0, N, K, tid);
-    ta.stash(lds_a, tid);
-    tb.stash(lds_b, tid);
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s) {
+#pragma unroll
+    for (int gi = 0; gi < kGroups; ++gi) issue_group(gi, lds_base + s * kStageBytes);
+    ta.advance();
+    tb.advance();
   }
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 3) * kLoads) : "memory");
   __syncthreads();
 
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < k_tiles;
-    if (more) {
-      ta.fetch(A, lda, m0, (kt + 1) * BK, M, K, tid);
-      tb.fetch(B, ldb, n0, (kt + 1) * BK, N, K, tid);
-    }
-    const uint16_t* la = lds_a + cur * ATile::kLdsElems;
-    const uint16_t* lb = lds_b + cur * BTile::kLdsElems;
+  uint4 fa[2][TM], fb[2][TN];
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      uint4 fa[TM], fb[TN];
+  for (int i = 0; i < TM; ++i)
+    fa[0][i] = ATile::frag(smem, wave_m * (BM / WM) + i * 32, 0, lane);
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
-        fa[i] = ATile::frag(la, wave_m * (BM / WM) + i * 32, kk, lane);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        fb[j] = BTile::frag(lb, wave_n * (BN / WN) + j * 32, kk, lane);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = Mma<T>::run(fa[i], fb[j], acc[i][j]);
-    }
-    if (more) {
-      ta.stash(lds_a + (cur ^ 1) * ATile::kLdsElems, tid);
-      tb.stash(lds_b + (cur ^ 1) * BTile::kLdsElems, tid);
-    }
-    __syncthreads();
-  }
+  for (int j = 0; j < TN; ++j)
+    fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 32, 0, lane);
 
-  // ---- epilogue: accumulator r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32]
+  int stage = 0;
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const int stage_next = stage + 1 == NS ? 0 : stage + 1;
+    const int stage_free = stage == 0 ? NS - 1 : stage - 1;
+    const uint32_t free_lds = lds_base + (uint32_t)stage_free * kStageBytes;
+    const uint16_t* la = smem + stage * kStageElems;
+    const uint16_t* lb = la + ATile::kBytes / 2;
+    const uint16_t* la_next = smem + stage_next * kStageElems;
+    const uint16_t* lb_next = la_next + ATile::kBytes / 2;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int cur = kk & 1;
+      const uint16_t* pa = kk + 1 < KK ? la : la_next;
+      const uint16_t* pb = kk + 1 < KK ? lb : lb_next;
+      const int kk_pre = kk + 1 < KK ? kk + 1 : 0;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          acc[i][j] = Mma<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
+          const int q = i * TN + j;
+          if (q < TM)
+            fa[cur ^ 1][q] = ATile::frag(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
+          else if (q < TM + TN)
+            fb[cur ^ 1][q - TM] =
+                BTile::frag(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
+          const int n = kk * TM * TN + q;
+          if (n % kEvery == kEvery / 2 && n / kEvery < kGroups)
+            issue_group(n / kEvery, free_lds);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    ta.advance();
+    tb.advance();
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 3) * kLoads) : "memory");
+    __syncthreads();
+    stage = stage_next;
+  }
+  // copies still in flight target LDS that nobody reads any more, but they must
+  // not outlive the block's LDS allocation
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  // ---- epilogue: accumulator r of lane l is
+  //      C[m = l%32][n = 8*(r/4) + 4*(l/32) + r%4] of its 32x32 block
   const T* bias = (MODE == GEMM_FWD && g.bias)
                       ? (const T*)g.bias + (int64_t)e * out_f : nullptr;
+  struct alignas(8) Out4 { T v[4]; };
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wave_n * (BN / WN) + j * 32 + (lane & 31);
-    if (n >= N) continue;
-    const float bv = bias ? Elem<T>::to_acc(bias[n]) : 0.f;
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wave_m * (BM / WM) + i * 32 + (lane & 31);
+    if (m >= M) continue;
+    T* crow = C + (int64_t)m * ldc;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int mb = m0 + wave_m * (BM / WM) + i * 32 + 4 * (lane >> 5);
+    for (int j = 0; j < TN; ++j) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = mb + 8 * (r / 4) + (r % 4);
-        if (m < M) C[(int64_t)m * ldc + n] = Elem<T>::from_acc(acc[i][j][r] + bv);
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
+        if (n >= N) continue;   // N is a multiple of 8: 4 columns are all in or all out
+        Out4 o;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          float v = acc[i][j][4 * q + c];
+          if (bias) v += Elem<T>::to_acc(bias[n + c]);
+          o.v[c] = Elem<T>::from_acc(v);
+        }
+        *reinterpret_cast<Out4*>(crow + n) = o;
       }
     }
   }
 }
 
 // ------------------------------------------------------------------ host side
-template <typename T, int BM, int BN, int BK, int WM, int WN, int MODE>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
 static int launch_cfg(const GemmArgs& g, hipStream_t s) {
-  constexpr int NT = WM * WN * 64;
-  using ATile = OperandTile<BM, BK, NT, MODE != GEMM_WGRAD>;
-  using BTile = OperandTile<BN, BK, NT, MODE == GEMM_FWD>;
-  constexpr size_t lds_bytes = 2 * (ATile::kLdsElems + BTile::kLdsElems) * sizeof(uint16_t);
-  auto kern = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, MODE>;
+  constexpr int NW = WM * WN;
+  constexpr int NT = NW * 64;
+  using ATile = DmaTile<BM, BK, NW, MODE != GEMM_WGRAD>;
+  using BTile = DmaTile<BN, BK, NW, MODE == GEMM_FWD>;
+  constexpr size_t lds_bytes = NS * (ATile::kBytes + BTile::kBytes);
+  static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
+  auto kern = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, NS, MODE>;
   static bool configured = false;  // attribute is per function, set once
   if (!configured) {
     FMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern,
@@ -295,14 +452,25 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   return FMOE_OK;
 }
 
+// Tile shape: 256x256 whenever that still yields at least two blocks per CU;
+// otherwise narrower tiles, so that a small problem is not left with a handful
+// of long-running blocks.  `g.tile` (1..3) overrides the choice for tuning.
 template <typename T, int MODE>
 static int launch_mode(const GemmArgs& g, hipStream_t s) {
-  // large tiles when the average expert fills them, small ones otherwise
-  bool large;
-  if (MODE == GEMM_WGRAD) large = g.in_feat >= 1024 && g.out_feat >= 1024;
-  else large = g.n_rows / g.n_expert >= 768;
-  if (large) return launch_cfg<T, 256, 256, 64, 2, 2, MODE>(g, s);
-  return launch_cfg<T, 128, 128, 64, 2, 2, MODE>(g, s);
+  const int64_t N = MODE == GEMM_FWD ? g.out_feat : g.in_feat;
+  auto tiles = [&](int bm, int bn) -> int64_t {
+    if (MODE == GEMM_WGRAD)
+      return (int64_t)g.n_expert * ceil_div(g.out_feat, bm) * ceil_div(g.in_feat, bn);
+    return (int64_t)ceil_div(g.n_rows, bm) * ceil_div(N, bn);
+  };
+  int pick = g.tile;
+  if (pick < 1 || pick > 3)
+    pick = tiles(256, 256) >= 512 ? 1 : (tiles(128, 256) >= 512 ? 2 : 3);
+  switch (pick) {
+    case 1: return launch_cfg<T, 256, 256, 32, 2, 2, 4, MODE>(g, s);
+    case 2: return launch_cfg<T, 128, 256, 32, 2, 2, 4, MODE>(g, s);
+    default: return launch_cfg<T, 128, 128, 32, 2, 2, 4, MODE>(g, s);
+  }
 }
 
 template <typename T>
@@ -318,6 +486,9 @@ bool gemm_mfma_supported(int mode, const GemmArgs& g, int dtype) {
   (void)mode;
   if (dtype != FMOE_BF16 && dtype != FMOE_F16) return false;
   if (g.in_feat % 8 != 0 || g.out_feat % 8 != 0) return false;
+  // tile-relative byte offsets are 32-bit: 256 rows of either feature size
+  if ((int64_t)g.in_feat * 512 >= (int64_t)kOutOfRange ||
+      (int64_t)g.out_feat * 512 >= (int64_t)kOutOfRange) return false;
   if (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.c) % 16 != 0) return false;
   return true;
 }
