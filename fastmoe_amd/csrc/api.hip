@@ -23,25 +23,39 @@ int set_error(int code, const char* fmt, ...) {
 
 // ------------------------------------------------------------ bias gradient
 // db[e][c] = sum over the rows of expert e of dy[r][c], fp32 accumulation
-// (fp64 for doubles).  Block = 32 column groups x 8 row lanes; a thread adds
-// VEC adjacent columns of every 8th row, then the 8 row lanes meet in LDS.
+// (fp64 for doubles).  Block = 16 column groups x 16 row lanes; a thread adds
+// VEC adjacent columns of every 16th row, four independent rows in flight per
+// step, then the 16 row lanes meet in LDS.  HBM-bound: reads dy once.
+constexpr int kBgCols = 16, kBgRows = 16, kBgUnroll = 4;
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void bias_grad_kernel(
+__global__ __launch_bounds__(kBgCols * kBgRows) void bias_grad_kernel(
     const T* __restrict__ dy, const int32_t* __restrict__ seg_off,
     T* __restrict__ db, int out_feat) {
   using acc_t = typename Elem<T>::acc_t;
   struct alignas(sizeof(T) * VEC) Pk { T v[VEC]; };
-  __shared__ acc_t part[8][32 * VEC + 1];
+  __shared__ acc_t part[kBgRows][kBgCols * VEC + 1];
   const int e = blockIdx.y;
-  const int cx = threadIdx.x % 32, ry = threadIdx.x / 32;
-  const int c0 = (blockIdx.x * 32 + cx) * VEC;
+  const int cx = threadIdx.x % kBgCols, ry = threadIdx.x / kBgCols;
+  const int c0 = (blockIdx.x * kBgCols + cx) * VEC;
   const int r_begin = seg_off[e], r_end = seg_off[e + 1];
   acc_t acc[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) acc[v] = 0;
   if (c0 < out_feat) {
-    for (int r = r_begin + ry; r < r_end; r += 8) {
-      const Pk p = *reinterpret_cast<const Pk*>(dy + (int64_t)r * out_feat + c0);
+    const T* col = dy + c0;
+    int r = r_begin + ry;
+    for (; r + (kBgUnroll - 1) * kBgRows < r_end; r += kBgUnroll * kBgRows) {
+      Pk p[kBgUnroll];
+#pragma unroll
+      for (int u = 0; u < kBgUnroll; ++u)
+        p[u] = *reinterpret_cast<const Pk*>(col + (int64_t)(r + u * kBgRows) * out_feat);
+#pragma unroll
+      for (int u = 0; u < kBgUnroll; ++u)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] += Elem<T>::to_acc(p[u].v[v]);
+    }
+    for (; r < r_end; r += kBgRows) {
+      const Pk p = *reinterpret_cast<const Pk*>(col + (int64_t)r * out_feat);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) acc[v] += Elem<T>::to_acc(p.v[v]);
     }
@@ -49,11 +63,11 @@ __global__ __launch_bounds__(256) void bias_grad_kernel(
 #pragma unroll
   for (int v = 0; v < VEC; ++v) part[ry][cx * VEC + v] = acc[v];
   __syncthreads();
-  for (int c = threadIdx.x; c < 32 * VEC; c += 256) {
+  for (int c = threadIdx.x; c < kBgCols * VEC; c += kBgCols * kBgRows) {
     acc_t s = 0;
 #pragma unroll
-    for (int y = 0; y < 8; ++y) s += part[y][c];
-    const int col = blockIdx.x * 32 * VEC + c;
+    for (int y = 0; y < kBgRows; ++y) s += part[y][c];
+    const int col = blockIdx.x * kBgCols * VEC + c;
     if (col < out_feat) db[(int64_t)e * out_feat + col] = Elem<T>::from_acc(s);
   }
 }
@@ -64,12 +78,12 @@ static int launch_bias_grad(const void* dy, const int32_t* seg_off, void* db,
   constexpr int kVec = 16 / sizeof(T);
   const bool vec = out_feat % kVec == 0 && ((uintptr_t)dy % 16) == 0;
   if (vec) {
-    dim3 grid(ceil_div(out_feat, 32 * kVec), n_expert);
-    hipLaunchKernelGGL((bias_grad_kernel<T, kVec>), grid, dim3(256), 0, s,
+    dim3 grid(ceil_div(out_feat, kBgCols * kVec), n_expert);
+    hipLaunchKernelGGL((bias_grad_kernel<T, kVec>), grid, dim3(kBgCols * kBgRows), 0, s,
                        (const T*)dy, seg_off, (T*)db, out_feat);
   } else {
-    dim3 grid(ceil_div(out_feat, 32), n_expert);
-    hipLaunchKernelGGL((bias_grad_kernel<T, 1>), grid, dim3(256), 0, s,
+    dim3 grid(ceil_div(out_feat, kBgCols), n_expert);
+    hipLaunchKernelGGL((bias_grad_kernel<T, 1>), grid, dim3(kBgCols * kBgRows), 0, s,
                        (const T*)dy, seg_off, (T*)db, out_feat);
   }
   FMOE_LAUNCH_CHECK("bias_grad");

@@ -391,6 +391,20 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   const T* bias = (MODE == GEMM_FWD && g.bias)
                       ? (const T*)g.bias + (int64_t)e * out_f : nullptr;
   struct alignas(8) Out4 { T v[4]; };
+  // this lane's bias values: 4 consecutive columns per (j, q), shared by all i
+  float bv[TN][4][4];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
+      Out4 b4;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) b4.v[c] = Elem<T>::from_acc(0.f);
+      if (bias && n < N) b4 = *reinterpret_cast<const Out4*>(bias + n);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) bv[j][q][c] = Elem<T>::to_acc(b4.v[c]);
+    }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int m = m0 + wave_m * (BM / WM) + i * 32 + (lane & 31);
@@ -404,11 +418,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
         if (n >= N) continue;   // N is a multiple of 8: 4 columns are all in or all out
         Out4 o;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          float v = acc[i][j][4 * q + c];
-          if (bias) v += Elem<T>::to_acc(bias[n + c]);
-          o.v[c] = Elem<T>::from_acc(v);
-        }
+        for (int c = 0; c < 4; ++c)
+          o.v[c] = Elem<T>::from_acc(acc[i][j][4 * q + c] + bv[j][q][c]);
         *reinterpret_cast<Out4*>(crow + n) = o;
       }
     }
