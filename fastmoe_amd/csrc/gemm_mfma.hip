@@ -382,47 +382,55 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
     __syncthreads();
     stage = stage_next;
   }
-  // copies still in flight target LDS that nobody reads any more, but they must
-  // not outlive the block's LDS allocation
+  // The zero-filled dummy slices are still landing in LDS: let them finish,
+  // then the whole LDS allocation is free to stage the output tile.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
 
   // ---- epilogue: accumulator r of lane l is
-  //      C[m = l%32][n = 8*(r/4) + 4*(l/32) + r%4] of its 32x32 block
+  //      C[m = l%32][n = 8*(r/4) + 4*(l/32) + r%4] of its 32x32 block.
+  // The tile goes through LDS (row-major, rows padded by 16 bytes so that the
+  // 8-byte writes of 32 rows spread over the banks) and leaves as 16-byte packs:
+  // one wave instruction then stores whole 512-byte row segments.
   const T* bias = (MODE == GEMM_FWD && g.bias)
                       ? (const T*)g.bias + (int64_t)e * out_f : nullptr;
   struct alignas(8) Out4 { T v[4]; };
-  // this lane's bias values: 4 consecutive columns per (j, q), shared by all i
-  float bv[TN][4][4];
+  constexpr int kLdc = BN + 8;   // elements per staged row
+  T* stage_c = reinterpret_cast<T*>(smem);
 #pragma unroll
-  for (int j = 0; j < TN; ++j)
+  for (int j = 0; j < TN; ++j) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int n = n0 + wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
-      Out4 b4;
+      const int col = wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias && n0 + col < N) {
+        const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
 #pragma unroll
-      for (int c = 0; c < 4; ++c) b4.v[c] = Elem<T>::from_acc(0.f);
-      if (bias && n < N) b4 = *reinterpret_cast<const Out4*>(bias + n);
+        for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
+      }
 #pragma unroll
-      for (int c = 0; c < 4; ++c) bv[j][q][c] = Elem<T>::to_acc(b4.v[c]);
-    }
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int m = m0 + wave_m * (BM / WM) + i * 32 + (lane & 31);
-    if (m >= M) continue;
-    T* crow = C + (int64_t)m * ldc;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
-        if (n >= N) continue;   // N is a multiple of 8: 4 columns are all in or all out
+      for (int i = 0; i < TM; ++i) {
+        const int row = wave_m * (BM / WM) + i * 32 + (lane & 31);
         Out4 o;
 #pragma unroll
         for (int c = 0; c < 4; ++c)
-          o.v[c] = Elem<T>::from_acc(acc[i][j][4 * q + c] + bv[j][q][c]);
-        *reinterpret_cast<Out4*>(crow + n) = o;
+          o.v[c] = Elem<T>::from_acc(acc[i][j][4 * q + c] + bv[c]);
+        *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
       }
     }
+  }
+  __syncthreads();
+  constexpr int kRowPacks = BN / 8;                  // 16-byte packs per tile row
+  constexpr int kPacksPerThread = BM * kRowPacks / NT;
+  static_assert((BM * kRowPacks) % NT == 0, "output tile must split evenly over the threads");
+#pragma unroll 4
+  for (int it = 0; it < kPacksPerThread; ++it) {
+    const int c = tid + it * NT;
+    const int row = c / kRowPacks, pk = c % kRowPacks;
+    const int m = m0 + row, n = n0 + pk * 8;
+    if (m < M && n < N)   // N is a multiple of 8: a pack is all in or all out
+      *reinterpret_cast<uint4*>(C + (int64_t)m * ldc + n) =
+          *reinterpret_cast<const uint4*>(stage_c + row * kLdc + pk * 8);
   }
 }
 
@@ -433,7 +441,9 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   constexpr int NT = NW * 64;
   using ATile = DmaTile<BM, BK, NW, MODE != GEMM_WGRAD>;
   using BTile = DmaTile<BN, BK, NW, MODE == GEMM_FWD>;
-  constexpr size_t lds_bytes = NS * (ATile::kBytes + BTile::kBytes);
+  constexpr size_t pipe_bytes = NS * (ATile::kBytes + BTile::kBytes);
+  constexpr size_t out_bytes = (size_t)BM * (BN + 8) * 2;   // staged output tile
+  constexpr size_t lds_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
   auto kern = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, NS, MODE>;
   static bool configured = false;  // attribute is per function, set once
