@@ -473,20 +473,32 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   return FMOE_OK;
 }
 
-// Tile shape: 256x256 whenever that still yields at least two blocks per CU;
-// otherwise narrower tiles, so that a small problem is not left with a handful
-// of long-running blocks.  `g.tile` (1..3) overrides the choice for tuning.
+// Tile shape by a small cost model: blocks run in rounds over the CUs that
+// take a block at a time (measured on MI355X: 248 blocks of a 256-thread,
+// >80 KiB-LDS kernel run concurrently), a tile costs a fixed prologue/epilogue
+// plus a per-K-slice time that depends on its shape (measured microseconds).
+// The shape with the least estimated time wins; `g.tile` (1..3) overrides the
+// choice for tuning.  Ragged experts add at most one partial tile each, which
+// the estimate ignores.
 template <typename T, int MODE>
 static int launch_mode(const GemmArgs& g, hipStream_t s) {
   const int64_t N = MODE == GEMM_FWD ? g.out_feat : g.in_feat;
-  auto tiles = [&](int bm, int bn) -> int64_t {
-    if (MODE == GEMM_WGRAD)
-      return (int64_t)g.n_expert * ceil_div(g.out_feat, bm) * ceil_div(g.in_feat, bn);
-    return (int64_t)ceil_div(g.n_rows, bm) * ceil_div(N, bn);
+  const int64_t K = MODE == GEMM_WGRAD ? g.n_rows / g.n_expert
+                                       : (MODE == GEMM_FWD ? g.in_feat : g.out_feat);
+  auto cost = [&](int bm, int bn, double us_per_slice, int blocks_per_cu) -> double {
+    const int64_t tiles = MODE == GEMM_WGRAD
+        ? (int64_t)g.n_expert * ceil_div(g.out_feat, bm) * ceil_div(g.in_feat, bn)
+        : (int64_t)ceil_div(g.n_rows, bm) * ceil_div(N, bn);
+    const int64_t slots = 248 * blocks_per_cu;
+    const double rounds = (double)((tiles + slots - 1) / slots);
+    return rounds * (8.0 + (double)ceil_div(K, 32) * us_per_slice * blocks_per_cu);
   };
   int pick = g.tile;
-  if (pick < 1 || pick > 3)
-    pick = tiles(256, 256) >= 512 ? 1 : (tiles(128, 256) >= 512 ? 2 : 3);
+  if (pick < 1 || pick > 3) {
+    const double c1 = cost(256, 256, 0.78, 1), c2 = cost(128, 256, 0.45, 1),
+                 c3 = cost(128, 128, 0.27, 2);
+    pick = c1 <= c2 && c1 <= c3 ? 1 : (c2 <= c3 ? 2 : 3);
+  }
   switch (pick) {
     case 1: return launch_cfg<T, 256, 256, 32, 2, 2, 4, MODE>(g, s);
     case 2: return launch_cfg<T, 128, 256, 32, 2, 2, 4, MODE>(g, s);
