@@ -204,6 +204,28 @@ struct DmaTile {
   }
 };
 
+// Tiles one XCD works on between two refills of its 32 CUs.
+constexpr int kXcdRun = 32;
+
+// Patch order over a rows x cols grid of tiles: bands of 16 rows, cut into
+// blocks of 8 columns, cut into patches of 4 rows that are walked column by
+// column.  32 consecutive numbers are a 4x8 patch (12 operand tiles for 32
+// products), 256 consecutive ones a 16x16 region.  Ragged edges shrink the
+// band, block or patch; the order stays a bijection.
+__device__ __forceinline__ void tile_order(int t, int rows, int cols, int& row, int& col) {
+  const int band = t / (16 * cols);
+  int r = t % (16 * cols);
+  const int band_rows = min(16, rows - band * 16);
+  const int blk = r / (band_rows * 8);
+  r %= band_rows * 8;
+  const int blk_cols = min(8, cols - blk * 8);
+  const int patch = r / (4 * blk_cols);
+  r %= 4 * blk_cols;
+  const int patch_rows = min(4, band_rows - patch * 4);
+  row = band * 16 + patch * 4 + r % patch_rows;
+  col = blk * 8 + r / patch_rows;
+}
+
 template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
                                                                 int tiles_n,
@@ -224,7 +246,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   static_assert(kLoads * (NS - 3) < 64, "vmcnt is a 6-bit counter");
 
   extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];  // [stage][A | B]
-  __shared__ int s_expert;
+  __shared__ int s_expert, s_tile, s_wave_sum[NW];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -233,26 +255,75 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   const int in_f = g.in_feat, out_f = g.out_feat;
 
   // ---- which tile is this block?
+  // The hardware hands consecutive workgroup ids to the 8 XCDs in turn, and
+  // each XCD has its own L2.  The live tiles are numbered 0..live-1 in the
+  // patch order of tile_order(); XCD x takes the runs [256 j + 32 x, +32) of
+  // that numbering (shorter runs when there are fewer than 256 tiles), one
+  // run per round of its 32 CUs, so the blocks that share
+  // an L2 work on a 4x8 patch and the whole chip on a 16x16 one.  Blocks past
+  // the live range sit at the end of the launch order and exit at once (idle
+  // blocks interleaved with live ones were measured to delay live blocks of
+  // the same XCD by a whole tile time).
   const int pid = blockIdx.x;
-  const int n_tile = pid % tiles_n;
-  int e, m_tile;
+  auto tile_number = [&](int live) {
+    const int run = min(kXcdRun, (live + 7) >> 3);  // fewer than 256 tiles: spread them
+    const int slot = pid >> 3;                      // position in this XCD's queue
+    return (slot / run) * (8 * run) + (pid & 7) * run + slot % run;
+  };
+  int e, m_tile, n_tile;
   if (MODE == GEMM_WGRAD) {
-    m_tile = (pid / tiles_n) % tiles_m;
-    e = pid / (tiles_n * tiles_m);
+    const int live = tiles_n * tiles_m * g.n_expert;
+    const int t = tile_number(live);
+    if (t >= live) return;
+    e = t / (tiles_n * tiles_m);
+    tile_order(t % (tiles_n * tiles_m), tiles_m, tiles_n, m_tile, n_tile);
   } else {
-    const int v = pid / tiles_n;  // virtual row tile
-    if (tid == 0) s_expert = -1;
+    // Expert x owns ceil(cnt_x / BM) row tiles, numbered one expert after the
+    // other.  Each thread sums the tiles of a contiguous run of experts, a
+    // block-wide scan turns the sums into first-tile numbers, and the thread
+    // whose run contains this block's row tile walks it to find the owner.
+    const int per_thread = (g.n_expert + NT - 1) / NT;
+    const int x_lo = min(tid * per_thread, g.n_expert);
+    const int x_hi = min(x_lo + per_thread, g.n_expert);
+    int mine = 0;
+    for (int x = x_lo; x < x_hi; ++x)
+      mine += (g.seg_off[x + 1] - g.seg_off[x] + BM - 1) / BM;
+    int incl = mine;  // inclusive scan inside the wave
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) s_wave_sum[wave] = incl;
     __syncthreads();
-    for (int x = tid; x < g.n_expert; x += NT) {
-      const int so = g.seg_off[x];
-      const int c = g.seg_off[x + 1] - so;
-      const int vs = so / BM + x;
-      if (v >= vs && v < vs + (c + BM - 1) / BM) s_expert = x;
+    int first = incl - mine, row_tiles = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; ++w2) {
+      const int ws = s_wave_sum[w2];
+      if (w2 < wave) first += ws;
+      row_tiles += ws;
+    }
+    const int live = row_tiles * tiles_n;
+    if (live == 0) return;
+    const int t = tile_number(live);
+    if (t >= live) return;  // the same for the whole block
+    int v;
+    tile_order(t, row_tiles, tiles_n, v, n_tile);
+    if (v >= first && v < first + mine) {
+      int f = first;
+      for (int x = x_lo; x < x_hi; ++x) {
+        const int tx = (g.seg_off[x + 1] - g.seg_off[x] + BM - 1) / BM;
+        if (v < f + tx) {
+          s_expert = x;
+          s_tile = v - f;
+          break;
+        }
+        f += tx;
+      }
     }
     __syncthreads();
     e = s_expert;
-    if (e < 0) return;  // nobody owns this virtual tile
-    m_tile = v - (g.seg_off[e] / BM + e);
+    m_tile = s_tile;
   }
   e = __builtin_amdgcn_readfirstlane(e);
   m_tile = __builtin_amdgcn_readfirstlane(m_tile);
@@ -464,6 +535,7 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
     tiles_m = virtual_row_tiles(g.n_rows, g.n_expert, BM);
     blocks = (int64_t)tiles_n * tiles_m;
   }
+  blocks = ceil_div(blocks, 8 * kXcdRun) * (8 * kXcdRun);  // whole runs for all 8 XCDs
   FMOE_REQUIRE(blocks < ((int64_t)1 << 31), FMOE_ERR_UNSUPPORTED,
                "grouped GEMM: too many tiles");
   if (blocks == 0) return FMOE_OK;
@@ -474,8 +546,8 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
 }
 
 // Tile shape by a small cost model: blocks run in rounds over the CUs that
-// take a block at a time (measured on MI355X: 248 blocks of a 256-thread,
-// >80 KiB-LDS kernel run concurrently), a tile costs a fixed prologue/epilogue
+// take a block at a time (256 CUs; live tiles come first in launch order, so a
+// round is really 256 wide), a tile costs a fixed prologue/epilogue
 // plus a per-K-slice time that depends on its shape (measured microseconds).
 // The shape with the least estimated time wins; `g.tile` (1..3) overrides the
 // choice for tuning.  Ragged experts add at most one partial tile each, which
@@ -489,7 +561,7 @@ static int launch_mode(const GemmArgs& g, hipStream_t s) {
     const int64_t tiles = MODE == GEMM_WGRAD
         ? (int64_t)g.n_expert * ceil_div(g.out_feat, bm) * ceil_div(g.in_feat, bn)
         : (int64_t)ceil_div(g.n_rows, bm) * ceil_div(N, bn);
-    const int64_t slots = 248 * blocks_per_cu;
+    const int64_t slots = 256 * blocks_per_cu;
     const double rounds = (double)((tiles + slots - 1) / slots);
     return rounds * (8.0 + (double)ceil_div(K, 32) * us_per_slice * blocks_per_cu);
   };
