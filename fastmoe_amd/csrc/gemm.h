@@ -24,11 +24,9 @@ struct GemmArgs {
   int tile;             // 0 = choose the tile shape automatically, 1..3 = force one
 };
 
-// Upper bound on the row tiles of a ragged product: sum_e ceil(cnt_e / BM) is at
-// most n_rows / BM + n_expert.  The scalar kernel uses it as a virtual index
-// space (expert e owns the tiles from seg_off[e] / BM + e on; the starts are
-// strictly increasing, so tiles that belong to nobody simply exit); the
-// matrix-core kernel numbers its tiles compactly and only sizes its grid by it.
+// Virtual row-tile index space of the scalar kernel: expert e owns the tiles
+// from seg_off[e] / BM + e on (the starts are strictly increasing, so tiles
+// that belong to nobody simply exit); n_rows / BM + n_expert bounds their number.
 inline int virtual_row_tiles(int64_t n_rows, int n_expert, int bm) {
   return (int)(n_rows / bm) + n_expert;
 }

@@ -23,8 +23,13 @@
 // descriptor's num_records and arrive as zeros, so there are no edge kernels
 // and no branches in the load path.
 //
-// Two LDS stages: the loads of K-slice t+1 are in flight while slice t feeds
-// the MFMAs; one barrier per slice.
+// NS (4) LDS stages of BK (32) values of K: two K-slices are always in flight
+// while one feeds the MFMAs; one barrier per slice.
+//
+// The rows of an expert are cut into BM-row tiles plus, for a remainder of at
+// most BM / 2 rows, 64-row tiles that cost a fraction of a BM tile, so a few
+// rows past a multiple of BM do not cost a whole tile.  Tiles are dealt to the
+// workgroups in an XCD-aware patch order.
 //
 // Operand roles follow cuda/parallel_linear.cuh:69-87,124-147 of the
 // reference; the per-expert cuBLAS loop there becomes a tile index space.
@@ -226,10 +231,11 @@ __device__ __forceinline__ void tile_order(int t, int rows, int cols, int& row, 
   col = blk * 8 + r / patch_rows;
 }
 
+// One output tile: rows [m0, m0 + BM) of expert e's row range (WGRAD: of its
+// out_feat x in_feat gradient) by columns [n_tile * BN, + BN).
 template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
-                                                                int tiles_n,
-                                                                int tiles_m) {
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, int e, int m0,
+                                          int n_tile) {
   constexpr int NW = WM * WN;
   constexpr int NT = NW * 64;
   constexpr bool A_KC = MODE != GEMM_WGRAD;
@@ -245,88 +251,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   constexpr int kGroups = ATile::kGroups + BTile::kGroups;   // asm groups per slice
   static_assert(kLoads * (NS - 3) < 64, "vmcnt is a 6-bit counter");
 
-  extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];  // [stage][A | B]
-  __shared__ int s_expert, s_tile, s_wave_sum[NW];
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave / WN, wave_n = wave % WN;
   const int in_f = g.in_feat, out_f = g.out_feat;
-
-  // ---- which tile is this block?
-  // The hardware hands consecutive workgroup ids to the 8 XCDs in turn, and
-  // each XCD has its own L2.  The live tiles are numbered 0..live-1 in the
-  // patch order of tile_order(); XCD x takes the runs [256 j + 32 x, +32) of
-  // that numbering (shorter runs when there are fewer than 256 tiles), one
-  // run per round of its 32 CUs, so the blocks that share
-  // an L2 work on a 4x8 patch and the whole chip on a 16x16 one.  Blocks past
-  // the live range sit at the end of the launch order and exit at once (idle
-  // blocks interleaved with live ones were measured to delay live blocks of
-  // the same XCD by a whole tile time).
-  const int pid = blockIdx.x;
-  auto tile_number = [&](int live) {
-    const int run = min(kXcdRun, (live + 7) >> 3);  // fewer than 256 tiles: spread them
-    const int slot = pid >> 3;                      // position in this XCD's queue
-    return (slot / run) * (8 * run) + (pid & 7) * run + slot % run;
-  };
-  int e, m_tile, n_tile;
-  if (MODE == GEMM_WGRAD) {
-    const int live = tiles_n * tiles_m * g.n_expert;
-    const int t = tile_number(live);
-    if (t >= live) return;
-    e = t / (tiles_n * tiles_m);
-    tile_order(t % (tiles_n * tiles_m), tiles_m, tiles_n, m_tile, n_tile);
-  } else {
-    // Expert x owns ceil(cnt_x / BM) row tiles, numbered one expert after the
-    // other.  Each thread sums the tiles of a contiguous run of experts, a
-    // block-wide scan turns the sums into first-tile numbers, and the thread
-    // whose run contains this block's row tile walks it to find the owner.
-    const int per_thread = (g.n_expert + NT - 1) / NT;
-    const int x_lo = min(tid * per_thread, g.n_expert);
-    const int x_hi = min(x_lo + per_thread, g.n_expert);
-    int mine = 0;
-    for (int x = x_lo; x < x_hi; ++x)
-      mine += (g.seg_off[x + 1] - g.seg_off[x] + BM - 1) / BM;
-    int incl = mine;  // inclusive scan inside the wave
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int up = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += up;
-    }
-    if (lane == 63) s_wave_sum[wave] = incl;
-    __syncthreads();
-    int first = incl - mine, row_tiles = 0;
-#pragma unroll
-    for (int w2 = 0; w2 < NW; ++w2) {
-      const int ws = s_wave_sum[w2];
-      if (w2 < wave) first += ws;
-      row_tiles += ws;
-    }
-    const int live = row_tiles * tiles_n;
-    if (live == 0) return;
-    const int t = tile_number(live);
-    if (t >= live) return;  // the same for the whole block
-    int v;
-    tile_order(t, row_tiles, tiles_n, v, n_tile);
-    if (v >= first && v < first + mine) {
-      int f = first;
-      for (int x = x_lo; x < x_hi; ++x) {
-        const int tx = (g.seg_off[x + 1] - g.seg_off[x] + BM - 1) / BM;
-        if (v < f + tx) {
-          s_expert = x;
-          s_tile = v - f;
-          break;
-        }
-        f += tx;
-      }
-    }
-    __syncthreads();
-    e = s_expert;
-    m_tile = s_tile;
-  }
   e = __builtin_amdgcn_readfirstlane(e);
-  m_tile = __builtin_amdgcn_readfirstlane(m_tile);
   const int row0 = __builtin_amdgcn_readfirstlane(g.seg_off[e]);
   const int cnt = __builtin_amdgcn_readfirstlane(g.seg_off[e + 1]) - row0;
 
@@ -349,7 +279,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
     B = (const uint16_t*)g.b + (int64_t)row0 * in_f;        ldb = in_f;
     C = (T*)g.c + (int64_t)e * out_f * in_f;                ldc = in_f;
   }
-  const int m0 = m_tile * BM, n0 = n_tile * BN;
+  m0 = __builtin_amdgcn_readfirstlane(m0);
+  const int n0 = __builtin_amdgcn_readfirstlane(n_tile) * BN;
   if (m0 >= M || n0 >= N) return;
   const int m_valid = min(BM, M - m0), n_valid = min(BN, N - n0);
 
@@ -505,6 +436,150 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   }
 }
 
+// Rows per remainder tile (see the kernel below).
+constexpr int kSmallRows = 64;
+
+// Whether tile shape BM x BN (4 waves) has a remainder shape kSmallRows x BN
+// (the 4 waves side by side) that the pipeline's interleaving plan accepts.
+template <int BM, int BN, int MODE>
+constexpr bool has_small_tiles() {
+  constexpr int tm = kSmallRows / 32, tn = BN / 4 / 32;
+  return MODE != GEMM_WGRAD && BM > kSmallRows && BN % 128 == 0 && tm + tn <= tm * tn;
+}
+
+// How expert rows are cut into tiles: `full` tiles of BM rows from row 0 on
+// and, behind them, `small` tiles of kSmallRows rows.  A remainder of more than
+// BM / 2 rows takes one more BM tile; a shorter one is covered by small tiles,
+// which cost a fraction of a BM tile instead of a whole one.
+template <int BM, bool SMALL>
+__device__ __forceinline__ void cut_rows(int cnt, int& full, int& small) {
+  if (!SMALL) {
+    full = (cnt + BM - 1) / BM;
+    small = 0;
+    return;
+  }
+  full = cnt / BM;
+  const int rem = cnt - full * BM;
+  small = 0;
+  if (rem > BM / 2) ++full;
+  else small = (rem + kSmallRows - 1) / kSmallRows;
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
+                                                                int tiles_n,
+                                                                int tiles_m) {
+  constexpr int NW = WM * WN;
+  constexpr int NT = NW * 64;
+  constexpr bool kSmall = has_small_tiles<BM, BN, MODE>();
+  static_assert(!kSmall || NW == 4, "remainder tiles put 4 waves side by side");
+  extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];  // [stage][A | B]
+  __shared__ int s_expert, s_row, s_wave_sum[2 * NW];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  // ---- which tile is this block?
+  // The hardware hands consecutive workgroup ids to the 8 XCDs in turn, and
+  // each XCD has its own L2.  The live tiles are numbered 0..live-1 in the
+  // patch order of tile_order(); XCD x takes the runs [256 j + 32 x, +32) of
+  // that numbering (shorter runs when there are fewer than 256 tiles), one
+  // run per round of its 32 CUs, so the blocks that share an L2 work on a 4x8
+  // patch and the whole chip on a 16x16 one.  Blocks past the live range sit
+  // at the end of the launch order and exit at once (idle blocks interleaved
+  // with live ones were measured to delay live blocks of the same XCD by a
+  // whole tile time).
+  const int pid = blockIdx.x;
+  auto tile_number = [&](int live) {
+    const int run = min(kXcdRun, (live + 7) >> 3);  // fewer than 256 tiles: spread them
+    const int slot = pid >> 3;                      // position in this XCD's queue
+    return (slot / run) * (8 * run) + (pid & 7) * run + slot % run;
+  };
+  if (MODE == GEMM_WGRAD) {
+    const int live = tiles_n * tiles_m * g.n_expert;
+    const int t = tile_number(live);
+    if (t >= live) return;
+    int m_tile, n_tile;
+    tile_order(t % (tiles_n * tiles_m), tiles_m, tiles_n, m_tile, n_tile);
+    gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, t / (tiles_n * tiles_m), m_tile * BM,
+                                                n_tile);
+    return;
+  }
+  // Ragged products.  The BM-row tiles of all experts are numbered first, one
+  // expert after the other, the remainder tiles behind them (long tiles start
+  // first).  Each thread cuts the rows of a contiguous run of experts, a
+  // block-wide scan turns the sums into first-tile numbers, and the thread
+  // whose run contains this block's row tile walks it to find the owner.
+  const int per_thread = (g.n_expert + NT - 1) / NT;
+  const int x_lo = min(tid * per_thread, g.n_expert);
+  const int x_hi = min(x_lo + per_thread, g.n_expert);
+  int mine_f = 0, mine_s = 0;
+  for (int x = x_lo; x < x_hi; ++x) {
+    int f, sm;
+    cut_rows<BM, kSmall>(g.seg_off[x + 1] - g.seg_off[x], f, sm);
+    mine_f += f;
+    mine_s += sm;
+  }
+  int incl_f = mine_f, incl_s = mine_s;  // inclusive scans inside the wave
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up_f = __shfl_up(incl_f, d, 64);
+    if (lane >= d) incl_f += up_f;
+    if (kSmall) {
+      const int up_s = __shfl_up(incl_s, d, 64);
+      if (lane >= d) incl_s += up_s;
+    }
+  }
+  if (lane == 63) {
+    s_wave_sum[wave] = incl_f;
+    s_wave_sum[NW + wave] = incl_s;
+  }
+  __syncthreads();
+  int first_f = incl_f - mine_f, first_s = incl_s - mine_s, rows_f = 0, rows_s = 0;
+#pragma unroll
+  for (int w2 = 0; w2 < NW; ++w2) {
+    const int wf = s_wave_sum[w2], ws = s_wave_sum[NW + w2];
+    if (w2 < wave) {
+      first_f += wf;
+      first_s += ws;
+    }
+    rows_f += wf;
+    rows_s += ws;
+  }
+  const int live_f = rows_f * tiles_n, live = live_f + rows_s * tiles_n;
+  if (live == 0) return;
+  const int t = tile_number(live);
+  if (t >= live) return;  // the same for the whole block
+  const bool small = t >= live_f;
+  int v, n_tile;
+  if (small) tile_order(t - live_f, rows_s, tiles_n, v, n_tile);
+  else tile_order(t, rows_f, tiles_n, v, n_tile);
+  const int first = small ? first_s : first_f, mine = small ? mine_s : mine_f;
+  if (v >= first && v < first + mine) {
+    int at = first;
+    for (int x = x_lo; x < x_hi; ++x) {
+      int f, sm;
+      cut_rows<BM, kSmall>(g.seg_off[x + 1] - g.seg_off[x], f, sm);
+      const int tx = small ? sm : f;
+      if (v < at + tx) {
+        s_expert = x;
+        s_row = small ? f * BM + (v - at) * kSmallRows : (v - at) * BM;
+        break;
+      }
+      at += tx;
+    }
+  }
+  __syncthreads();
+  if constexpr (kSmall) {
+    if (small) {
+      gemm_tile<T, kSmallRows, BN, BK, 1, NW, NS, MODE>(g, smem, s_expert, s_row, n_tile);
+      return;
+    }
+  }
+  gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, s_expert, s_row, n_tile);
+}
+
 // ------------------------------------------------------------------ host side
 template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
 static int launch_cfg(const GemmArgs& g, hipStream_t s) {
@@ -532,7 +607,11 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
     blocks = (int64_t)tiles_n * tiles_m * g.n_expert;
   } else {
     tiles_n = ceil_div(MODE == GEMM_FWD ? g.out_feat : g.in_feat, BN);
-    tiles_m = virtual_row_tiles(g.n_rows, g.n_expert, BM);
+    // at most n_rows / BM whole tiles plus, per expert, one more BM tile or
+    // the small tiles of half a BM tile
+    constexpr int kPerExpert = has_small_tiles<BM, BN, MODE>() && BM / 2 > kSmallRows
+                                   ? BM / 2 / kSmallRows : 1;
+    tiles_m = (int)(g.n_rows / BM) + g.n_expert * kPerExpert;
     blocks = (int64_t)tiles_n * tiles_m;
   }
   blocks = ceil_div(blocks, 8 * kXcdRun) * (8 * kXcdRun);  // whole runs for all 8 XCDs

@@ -75,6 +75,16 @@ def test_matrix_core_large_tiles_and_dead_rows(dt):
     _run([1000, 0, 1531, 800], 512, 1024, DTYPES[dt], True, path=0, extra_rows=37)
 
 
+@pytest.mark.parametrize("n_expert", [257, 600, 4096])
+def test_matrix_core_many_experts(n_expert):
+    # more experts than threads in a block: every thread of the tile search owns
+    # a run of experts; two thirds of them are empty
+    rng = np.random.default_rng(n_expert)
+    counts = (rng.integers(0, 30, n_expert) * (rng.random(n_expert) < 0.34)).tolist()
+    counts[-1] = 5
+    _run(counts, 32, 48, torch.bfloat16, True, path=0, extra_rows=3)
+
+
 def test_device_side_counts_and_seg_off_upload():
     from fastmoe_amd import fmoe_cuda
 
