@@ -190,6 +190,18 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
   FMOE_REQUIRE(n_rows == 0 || dy != nullptr, FMOE_ERR_INVALID,
                "grouped_linear_bwd: dy is null");
   hipStream_t s = (hipStream_t)stream;
+  if (dx && dw && n_rows > 0 && g_gemm_path == 0) {
+    FMOE_REQUIRE(w != nullptr && x != nullptr, FMOE_ERR_INVALID,
+                 "grouped_linear_bwd: w or x is null");
+    GemmArgs gd{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
+    GemmArgs gw{dy, x, dw, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
+    if (gemm_mfma_supported(GEMM_DGRAD, gd, dtype) && gemm_mfma_supported(GEMM_WGRAD, gw, dtype)) {
+      rc = launch_gemm_mfma_bwd(gd, gw, dtype, s);
+      if (rc) return rc;
+      dx = nullptr;  // both products are under way
+      dw = nullptr;
+    }
+  }
   if (dx && n_rows > 0) {
     FMOE_REQUIRE(w != nullptr, FMOE_ERR_INVALID, "grouped_linear_bwd: w is null");
     GemmArgs g{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};

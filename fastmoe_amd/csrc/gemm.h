@@ -39,5 +39,8 @@ int launch_gemm_simt(int mode, const GemmArgs& g, int dtype, hipStream_t s);
 // kernel).
 bool gemm_mfma_supported(int mode, const GemmArgs& g, int dtype);
 int launch_gemm_mfma(int mode, const GemmArgs& g, int dtype, hipStream_t s);
+// dX (gd: a = dY, b = W, c = dX) and dW (gw: a = dY, b = X, c = dW) of one
+// grouped linear, in one launch where the tile shapes allow it.
+int launch_gemm_mfma_bwd(const GemmArgs& gd, const GemmArgs& gw, int dtype, hipStream_t s);
 
 }  // namespace fmoe

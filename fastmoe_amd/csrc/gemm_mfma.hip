@@ -465,40 +465,113 @@ __device__ __forceinline__ void cut_rows(int cnt, int& full, int& small) {
   else small = (rem + kSmallRows - 1) / kSmallRows;
 }
 
+// Position of a workgroup in the order in which tiles are handed out.
+// The hardware gives consecutive workgroup ids to the 8 XCDs in turn, and each
+// XCD has its own L2.  The live tiles are numbered 0..live-1 so that
+// neighbours share operands (tile_order()); XCD x takes the runs
+// [256 j + 32 x, +32) of that numbering (shorter runs when there are fewer than
+// 256 tiles), one run per round of its 32 CUs, so the blocks that share an L2
+// work on a 4x8 patch and the whole chip on a 16x16 one.  Blocks past the live
+// range sit at the end of the launch order and exit at once (idle blocks
+// interleaved with live ones were measured to delay live blocks of the same
+// XCD by a whole tile time).
+__device__ __forceinline__ int tile_number(int pid, int live) {
+  const int run = max(1, min(kXcdRun, (live + 7) >> 3));  // fewer than 256 tiles: spread them
+  const int slot = pid >> 3;                      // position in this XCD's queue
+  return (slot / run) * (8 * run) + (pid & 7) * run + slot % run;
+}
+
+// Row tiles of a ragged product.  The BM-row tiles of all experts are numbered
+// first, one expert after the other, the remainder tiles behind them.  Each
+// thread cuts the rows of a contiguous run of experts and a block-wide scan
+// turns the sums into first-tile numbers; the thread whose run contains a
+// given row tile walks the run to find its owner.
+template <int BM, bool SMALL, int NW>
+struct RowTiles {
+  int x_lo, x_hi;          // this thread's run of experts
+  int mine_f, mine_s;      // BM-row / remainder tiles in the run
+  int first_f, first_s;    // number of the run's first tile of either kind
+  int rows_f, rows_s;      // totals over all experts
+
+  // Contains a __syncthreads(); s_wave_sum has 2 * NW entries.
+  __device__ __forceinline__ void scan(const int32_t* seg_off, int n_expert, int* s_wave_sum) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int per_thread = (n_expert + NW * 64 - 1) / (NW * 64);
+    x_lo = min(tid * per_thread, n_expert);
+    x_hi = min(x_lo + per_thread, n_expert);
+    mine_f = mine_s = 0;
+    for (int x = x_lo; x < x_hi; ++x) {
+      int f, sm;
+      cut_rows<BM, SMALL>(seg_off[x + 1] - seg_off[x], f, sm);
+      mine_f += f;
+      mine_s += sm;
+    }
+    int incl_f = mine_f, incl_s = mine_s;  // inclusive scans inside the wave
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up_f = __shfl_up(incl_f, d, 64);
+      if (lane >= d) incl_f += up_f;
+      if (SMALL) {
+        const int up_s = __shfl_up(incl_s, d, 64);
+        if (lane >= d) incl_s += up_s;
+      }
+    }
+    if (lane == 63) {
+      s_wave_sum[wave] = incl_f;
+      s_wave_sum[NW + wave] = incl_s;
+    }
+    __syncthreads();
+    first_f = incl_f - mine_f;
+    first_s = incl_s - mine_s;
+    rows_f = rows_s = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; ++w2) {
+      const int wf = s_wave_sum[w2], ws = s_wave_sum[NW + w2];
+      if (w2 < wave) {
+        first_f += wf;
+        first_s += ws;
+      }
+      rows_f += wf;
+      rows_s += ws;
+    }
+  }
+
+  // The owner of row tile v (of the remainder kind if `small`) stores the
+  // expert and the tile's first row inside the expert; the caller then syncs.
+  __device__ __forceinline__ void find(const int32_t* seg_off, int v, bool small,
+                                       int* s_expert, int* s_row) const {
+    const int first = small ? first_s : first_f, mine = small ? mine_s : mine_f;
+    if (v < first || v >= first + mine) return;
+    int at = first;
+    for (int x = x_lo; x < x_hi; ++x) {
+      int f, sm;
+      cut_rows<BM, SMALL>(seg_off[x + 1] - seg_off[x], f, sm);
+      const int tx = small ? sm : f;
+      if (v < at + tx) {
+        *s_expert = x;
+        *s_row = small ? f * BM + (v - at) * kSmallRows : (v - at) * BM;
+        return;
+      }
+      at += tx;
+    }
+  }
+};
+
+// One of the three products.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
                                                                 int tiles_n,
                                                                 int tiles_m) {
   constexpr int NW = WM * WN;
-  constexpr int NT = NW * 64;
   constexpr bool kSmall = has_small_tiles<BM, BN, MODE>();
   static_assert(!kSmall || NW == 4, "remainder tiles put 4 waves side by side");
   extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];  // [stage][A | B]
   __shared__ int s_expert, s_row, s_wave_sum[2 * NW];
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-
-  // ---- which tile is this block?
-  // The hardware hands consecutive workgroup ids to the 8 XCDs in turn, and
-  // each XCD has its own L2.  The live tiles are numbered 0..live-1 in the
-  // patch order of tile_order(); XCD x takes the runs [256 j + 32 x, +32) of
-  // that numbering (shorter runs when there are fewer than 256 tiles), one
-  // run per round of its 32 CUs, so the blocks that share an L2 work on a 4x8
-  // patch and the whole chip on a 16x16 one.  Blocks past the live range sit
-  // at the end of the launch order and exit at once (idle blocks interleaved
-  // with live ones were measured to delay live blocks of the same XCD by a
-  // whole tile time).
   const int pid = blockIdx.x;
-  auto tile_number = [&](int live) {
-    const int run = min(kXcdRun, (live + 7) >> 3);  // fewer than 256 tiles: spread them
-    const int slot = pid >> 3;                      // position in this XCD's queue
-    return (slot / run) * (8 * run) + (pid & 7) * run + slot % run;
-  };
   if (MODE == GEMM_WGRAD) {
     const int live = tiles_n * tiles_m * g.n_expert;
-    const int t = tile_number(live);
+    const int t = tile_number(pid, live);
     if (t >= live) return;
     int m_tile, n_tile;
     tile_order(t % (tiles_n * tiles_m), tiles_m, tiles_n, m_tile, n_tile);
@@ -506,70 +579,17 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
                                                 n_tile);
     return;
   }
-  // Ragged products.  The BM-row tiles of all experts are numbered first, one
-  // expert after the other, the remainder tiles behind them (long tiles start
-  // first).  Each thread cuts the rows of a contiguous run of experts, a
-  // block-wide scan turns the sums into first-tile numbers, and the thread
-  // whose run contains this block's row tile walks it to find the owner.
-  const int per_thread = (g.n_expert + NT - 1) / NT;
-  const int x_lo = min(tid * per_thread, g.n_expert);
-  const int x_hi = min(x_lo + per_thread, g.n_expert);
-  int mine_f = 0, mine_s = 0;
-  for (int x = x_lo; x < x_hi; ++x) {
-    int f, sm;
-    cut_rows<BM, kSmall>(g.seg_off[x + 1] - g.seg_off[x], f, sm);
-    mine_f += f;
-    mine_s += sm;
-  }
-  int incl_f = mine_f, incl_s = mine_s;  // inclusive scans inside the wave
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int up_f = __shfl_up(incl_f, d, 64);
-    if (lane >= d) incl_f += up_f;
-    if (kSmall) {
-      const int up_s = __shfl_up(incl_s, d, 64);
-      if (lane >= d) incl_s += up_s;
-    }
-  }
-  if (lane == 63) {
-    s_wave_sum[wave] = incl_f;
-    s_wave_sum[NW + wave] = incl_s;
-  }
-  __syncthreads();
-  int first_f = incl_f - mine_f, first_s = incl_s - mine_s, rows_f = 0, rows_s = 0;
-#pragma unroll
-  for (int w2 = 0; w2 < NW; ++w2) {
-    const int wf = s_wave_sum[w2], ws = s_wave_sum[NW + w2];
-    if (w2 < wave) {
-      first_f += wf;
-      first_s += ws;
-    }
-    rows_f += wf;
-    rows_s += ws;
-  }
-  const int live_f = rows_f * tiles_n, live = live_f + rows_s * tiles_n;
+  RowTiles<BM, kSmall, NW> rows;
+  rows.scan(g.seg_off, g.n_expert, s_wave_sum);
+  const int live_f = rows.rows_f * tiles_n, live = live_f + rows.rows_s * tiles_n;
   if (live == 0) return;
-  const int t = tile_number(live);
+  const int t = tile_number(pid, live);
   if (t >= live) return;  // the same for the whole block
-  const bool small = t >= live_f;
+  const bool small = t >= live_f;  // BM-row tiles start first: they take longer
   int v, n_tile;
-  if (small) tile_order(t - live_f, rows_s, tiles_n, v, n_tile);
-  else tile_order(t, rows_f, tiles_n, v, n_tile);
-  const int first = small ? first_s : first_f, mine = small ? mine_s : mine_f;
-  if (v >= first && v < first + mine) {
-    int at = first;
-    for (int x = x_lo; x < x_hi; ++x) {
-      int f, sm;
-      cut_rows<BM, kSmall>(g.seg_off[x + 1] - g.seg_off[x], f, sm);
-      const int tx = small ? sm : f;
-      if (v < at + tx) {
-        s_expert = x;
-        s_row = small ? f * BM + (v - at) * kSmallRows : (v - at) * BM;
-        break;
-      }
-      at += tx;
-    }
-  }
+  if (small) tile_order(t - live_f, rows.rows_s, tiles_n, v, n_tile);
+  else tile_order(t, rows.rows_f, tiles_n, v, n_tile);
+  rows.find(g.seg_off, v, small, &s_expert, &s_row);
   __syncthreads();
   if constexpr (kSmall) {
     if (small) {
@@ -578,6 +598,57 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
     }
   }
   gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, s_expert, s_row, n_tile);
+}
+
+// Both gradient products of one grouped linear in one launch: the BM-row
+// tiles of dX = dY W first, then the tiles of dW = dY^T X and the remainder
+// tiles of dX, whichever of the two kinds takes longer first (`small_first`).
+// The tail of one product overlaps the head of the next instead of leaving CUs
+// idle between two launches.  gd / gw are the arguments the two products
+// would get on their own.
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NS>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, GemmArgs gw,
+                                                               int tiles_n_d, int tiles_n_w,
+                                                               int tiles_m_w, int small_first) {
+  constexpr int NW = WM * WN;
+  constexpr bool kSmall = has_small_tiles<BM, BN, GEMM_DGRAD>();
+  static_assert(!kSmall || NW == 4, "remainder tiles put 4 waves side by side");
+  extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];
+  __shared__ int s_expert, s_row, s_wave_sum[2 * NW];
+
+  RowTiles<BM, kSmall, NW> rows;
+  rows.scan(gd.seg_off, gd.n_expert, s_wave_sum);
+  const int live_d = rows.rows_f * tiles_n_d, live_s = rows.rows_s * tiles_n_d;
+  const int per_expert_w = tiles_n_w * tiles_m_w;
+  const int live_w = per_expert_w * gw.n_expert;
+  const int live = live_d + live_w + live_s;
+  if (live == 0) return;
+  const int t = tile_number(blockIdx.x, live);
+  if (t >= live) return;  // the same for the whole block
+  // [0, live_d): dX tiles; then the dW range and the remainder range
+  const int w_begin = live_d + (small_first ? live_s : 0);
+  const int s_begin = live_d + (small_first ? 0 : live_w);
+  if (t >= w_begin && t < w_begin + live_w) {
+    const int tw = t - w_begin;
+    int m_tile, n_tile;
+    tile_order(tw % per_expert_w, tiles_m_w, tiles_n_w, m_tile, n_tile);
+    gemm_tile<T, BM, BN, BK, WM, WN, NS, GEMM_WGRAD>(gw, smem, tw / per_expert_w, m_tile * BM,
+                                                      n_tile);
+    return;
+  }
+  const bool small = t >= live_d;
+  int v, n_tile;
+  if (small) tile_order(t - s_begin, rows.rows_s, tiles_n_d, v, n_tile);
+  else tile_order(t, rows.rows_f, tiles_n_d, v, n_tile);
+  rows.find(gd.seg_off, v, small, &s_expert, &s_row);
+  __syncthreads();
+  if constexpr (kSmall) {
+    if (small) {
+      gemm_tile<T, kSmallRows, BN, BK, 1, NW, NS, GEMM_DGRAD>(gd, smem, s_expert, s_row, n_tile);
+      return;
+    }
+  }
+  gemm_tile<T, BM, BN, BK, WM, WN, NS, GEMM_DGRAD>(gd, smem, s_expert, s_row, n_tile);
 }
 
 // ------------------------------------------------------------------ host side
@@ -631,8 +702,9 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
 // The shape with the least estimated time wins; `g.tile` (1..3) overrides the
 // choice for tuning.  Ragged experts add at most one partial tile each, which
 // the estimate ignores.
-template <typename T, int MODE>
-static int launch_mode(const GemmArgs& g, hipStream_t s) {
+template <int MODE>
+static int pick_tile(const GemmArgs& g) {
+  if (g.tile >= 1 && g.tile <= 3) return g.tile;
   const int64_t N = MODE == GEMM_FWD ? g.out_feat : g.in_feat;
   const int64_t K = MODE == GEMM_WGRAD ? g.n_rows / g.n_expert
                                        : (MODE == GEMM_FWD ? g.in_feat : g.out_feat);
@@ -644,13 +716,14 @@ static int launch_mode(const GemmArgs& g, hipStream_t s) {
     const double rounds = (double)((tiles + slots - 1) / slots);
     return rounds * (8.0 + (double)ceil_div(K, 32) * us_per_slice * blocks_per_cu);
   };
-  int pick = g.tile;
-  if (pick < 1 || pick > 3) {
-    const double c1 = cost(256, 256, 0.78, 1), c2 = cost(128, 256, 0.45, 1),
-                 c3 = cost(128, 128, 0.27, 2);
-    pick = c1 <= c2 && c1 <= c3 ? 1 : (c2 <= c3 ? 2 : 3);
-  }
-  switch (pick) {
+  const double c1 = cost(256, 256, 0.78, 1), c2 = cost(128, 256, 0.45, 1),
+               c3 = cost(128, 128, 0.27, 2);
+  return c1 <= c2 && c1 <= c3 ? 1 : (c2 <= c3 ? 2 : 3);
+}
+
+template <typename T, int MODE>
+static int launch_mode(const GemmArgs& g, hipStream_t s) {
+  switch (pick_tile<MODE>(g)) {
     case 1: return launch_cfg<T, 256, 256, 32, 2, 2, 4, MODE>(g, s);
     case 2: return launch_cfg<T, 128, 256, 32, 2, 2, 4, MODE>(g, s);
     default: return launch_cfg<T, 128, 128, 32, 2, 2, 4, MODE>(g, s);
@@ -666,6 +739,45 @@ static int launch_t(int mode, const GemmArgs& g, hipStream_t s) {
   }
 }
 
+// dX and dW in one launch when both products would use the 256x256 tiles
+// anyway; otherwise one launch each.
+template <typename T>
+static int launch_bwd_t(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
+  if (pick_tile<GEMM_DGRAD>(gd) != 1 || pick_tile<GEMM_WGRAD>(gw) != 1) {
+    const int rc = launch_mode<T, GEMM_DGRAD>(gd, s);
+    return rc ? rc : launch_mode<T, GEMM_WGRAD>(gw, s);
+  }
+  constexpr int BM = 256, BN = 256, BK = 32, WM = 2, WN = 2, NS = 4, NT = WM * WN * 64;
+  constexpr size_t pipe_bytes = (size_t)NS * (BM + BN) * BK * 2;
+  constexpr size_t out_bytes = (size_t)BM * (BN + 8) * 2;
+  constexpr size_t lds_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
+  static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
+  auto kern = gemm_bwd_kernel<T, BM, BN, BK, WM, WN, NS>;
+  static bool configured = false;  // attribute is per function, set once
+  if (!configured) {
+    FMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds_bytes));
+    configured = true;
+  }
+  const int tiles_n_d = ceil_div(gd.in_feat, BN);
+  const int tiles_n_w = ceil_div(gw.in_feat, BN), tiles_m_w = ceil_div(gw.out_feat, BM);
+  constexpr int kPerExpert = BM / 2 / kSmallRows;  // see launch_cfg
+  int64_t blocks = (int64_t)tiles_n_d * (gd.n_rows / BM + (int64_t)gd.n_expert * kPerExpert) +
+                   (int64_t)tiles_n_w * tiles_m_w * gw.n_expert;
+  blocks = ceil_div(blocks, 8 * kXcdRun) * (8 * kXcdRun);
+  FMOE_REQUIRE(blocks < ((int64_t)1 << 31), FMOE_ERR_UNSUPPORTED,
+               "grouped GEMM: too many tiles");
+  // a remainder tile walks out_feat values of K at about 0.34 us per 32, a dW
+  // tile the rows of one expert at about 0.78 us per 32 (measured)
+  const int small_first =
+      0.34 * gd.out_feat > 0.78 * (double)(gd.n_rows / gd.n_expert) ? 1 : 0;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NT), lds_bytes, s, gd, gw, tiles_n_d,
+                     tiles_n_w, tiles_m_w, small_first);
+  FMOE_LAUNCH_CHECK("gemm_bwd");
+  return FMOE_OK;
+}
+
 bool gemm_mfma_supported(int mode, const GemmArgs& g, int dtype) {
   (void)mode;
   if (dtype != FMOE_BF16 && dtype != FMOE_F16) return false;
@@ -675,6 +787,13 @@ bool gemm_mfma_supported(int mode, const GemmArgs& g, int dtype) {
       (int64_t)g.out_feat * 512 >= (int64_t)kOutOfRange) return false;
   if (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.c) % 16 != 0) return false;
   return true;
+}
+
+int launch_gemm_mfma_bwd(const GemmArgs& gd, const GemmArgs& gw, int dtype, hipStream_t s) {
+  if (!gemm_mfma_supported(GEMM_DGRAD, gd, dtype) || !gemm_mfma_supported(GEMM_WGRAD, gw, dtype))
+    return set_error(FMOE_ERR_UNSUPPORTED, "grouped GEMM: shape not MFMA-aligned");
+  if (dtype == FMOE_BF16) return launch_bwd_t<__hip_bfloat16>(gd, gw, s);
+  return launch_bwd_t<__half>(gd, gw, s);
 }
 
 int launch_gemm_mfma(int mode, const GemmArgs& g, int dtype, hipStream_t s) {
