@@ -10,7 +10,7 @@ namespace fmoe {
 
 static thread_local char g_err[512] = "";
 static int g_gemm_path = 0;  // 0 = automatic, 1 = scalar kernel only
-// tuning aid: FMOE_GEMM_TILE=1..3 forces one MFMA tile shape (0 / unset = automatic)
+// tuning aid: FMOE_GEMM_TILE=1..4 forces one MFMA tile configuration (0 / unset = automatic)
 static int g_tile = getenv("FMOE_GEMM_TILE") ? atoi(getenv("FMOE_GEMM_TILE")) : 0;
 
 int set_error(int code, const char* fmt, ...) {

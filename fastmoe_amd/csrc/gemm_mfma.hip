@@ -33,6 +33,8 @@
 //
 // Operand roles follow cuda/parallel_linear.cuh:69-87,124-147 of the
 // reference; the per-expert cuBLAS loop there becomes a tile index space.
+#include <type_traits>
+
 #include "gemm.h"
 
 namespace fmoe {
@@ -60,25 +62,19 @@ template <> struct Mma<__half> {
 
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any num_records used here
 constexpr int kRsrcFlags = 0x00020000;         // raw buffer, 32-bit data format
-constexpr int kImmSpan = 3072;                 // largest immediate offset used (3 KiB)
 
 // One operand tile of R rows (the M or N index) by BK values of K.
 // KC == true : memory is [row][k] (k contiguous), LDS is [row][BK].
 // KC == false: memory is [k][row] (row contiguous), LDS is [k][R].
 //
-// A wave copies kPerWave consecutive 1 KiB blocks of the tile per K-slice, in
-// groups of up to four instructions that share one M0 (LDS base) and step
-// through the blocks with the instruction's immediate offset.  The hardware
-// adds that immediate to the global offset as well, so the descriptor base is
-// set kImmSpan bytes low and every lane offset carries the difference.
+// A wave copies kPerWave consecutive 1 KiB blocks of the tile per K-slice, one
+// buffer_load_dwordx4 ... lds each.
 template <int R, int BK, int NW, bool KC>
 struct DmaTile {
   static constexpr int kBytes = R * BK * 2;
   static constexpr int kBlocks = kBytes / 1024;     // one wave instruction each
   static constexpr int kPerWave = kBlocks / NW;
-  static constexpr int kGroup = kPerWave >= 4 ? 4 : kPerWave;
-  static constexpr int kGroups = kPerWave / kGroup;
-  static_assert(kBlocks % NW == 0 && kPerWave % kGroup == 0, "tile must split evenly");
+  static_assert(kBlocks % NW == 0 && kPerWave >= 1, "tile must split evenly");
   static_assert(BK == 64 || BK == 32, "swizzles below assume 128- or 64-byte [row][BK] rows");
   static constexpr int kRowPacks = R / 8;           // packs per [k] row (KC == false)
   static constexpr int kKPacks = BK / 8;            // packs per [row] row (KC == true)
@@ -88,15 +84,20 @@ struct DmaTile {
   __device__ static __forceinline__ int row_swizzle(int row) {
     return BK == 64 ? ((row & 7) ^ ((row >> 3) & 1)) : ((row >> 2) & 3);
   }
+  // K offset (elements) inside the slice of the pack lane `lane` copies in
+  // block b (KC only).
+  __device__ static __forceinline__ int pack_k(int b, int lane) {
+    const int row = b * (64 / kKPacks) + lane / kKPacks;
+    return ((lane % kKPacks) ^ row_swizzle(row)) * 8;
+  }
 
-  // per lane
-  uint32_t voff[kPerWave];  // byte offset of this lane's pack (+ immediate compensation)
-  int kpack[kPerWave];      // KC: K offset (elements) of the pack inside the slice
+  // per lane: byte offset of this lane's pack in each of the wave's blocks
+  uint32_t voff[kPerWave];
   // per wave (scalar registers)
-  uint32_t base_lo, base_hi;  // descriptor base of the current slice, kImmSpan low
-  int remaining;              // bytes from the slice origin to the end of the valid data
-  int step;                   // bytes between consecutive slices
-  int k_left;                 // K values from the slice start to the end of K
+  i32x4_t rsrc;       // buffer descriptor of the current slice; num_records ends the valid data
+  int remaining;      // bytes from the slice origin to the end of the valid data
+  int step;           // bytes between consecutive slices
+  int k_left;         // K values from the slice start to the end of K
 
   // origin: element (row 0, k 0) of the tile; ld: elements between rows (KC)
   // or between consecutive k (not KC); r_valid rows and k_total values of K
@@ -106,22 +107,15 @@ struct DmaTile {
 #pragma unroll
     for (int i = 0; i < kPerWave; ++i) {
       const int b = wave * kPerWave + i;
-      const uint32_t comp = (uint32_t)(kImmSpan - (i % kGroup) * 1024);
       if (KC) {
         const int row = b * (64 / kKPacks) + lane / kKPacks;
-        const int kc = (lane % kKPacks) ^ row_swizzle(row);
-        voff[i] = (uint32_t)(row * ld + kc * 8) * 2u + comp;
-        kpack[i] = kc * 8;
+        voff[i] = (uint32_t)(row * ld + pack_k(b, lane)) * 2u;
       } else {
         const int k = b * (64 / kRowPacks) + lane / kRowPacks;
         const int rc = (lane % kRowPacks) ^ ((k & 3) << 1);
-        voff[i] = rc * 8 < r_valid ? (uint32_t)(k * ld + rc * 8) * 2u + comp : kOutOfRange;
-        kpack[i] = 0;
+        voff[i] = rc * 8 < r_valid ? (uint32_t)(k * ld + rc * 8) * 2u : kOutOfRange;
       }
     }
-    const uint64_t p = (uint64_t)origin - kImmSpan;
-    base_lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
-    base_hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32));
     // everything past the ragged edge is beyond num_records and reads as zero
     remaining = KC ? ((r_valid - 1) * ld + k_total) * 2
                    : ((k_total - 1) * ld + r_span) * 2;
@@ -129,57 +123,49 @@ struct DmaTile {
     remaining = __builtin_amdgcn_readfirstlane(remaining);
     step = __builtin_amdgcn_readfirstlane((KC ? BK : BK * ld) * 2);
     k_left = k_total;
+    const uint64_t p = (uint64_t)origin;
+    rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    rsrc[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32) & 0xffff);  // stride 0
+    rsrc[2] = max(remaining, 0);
+    rsrc[3] = kRsrcFlags;
+    mask_k_tail(wave, lane);
+  }
+
+  // [row][k] memory cannot end a row early through num_records: in the one
+  // slice that holds the end of K, the packs past it are pointed out of range
+  // for good (the slices after it are empty anyway).
+  __device__ __forceinline__ void mask_k_tail(int wave, int lane) {
+    if (KC && k_left < BK) {
+#pragma unroll
+      for (int i = 0; i < kPerWave; ++i)
+        if (pack_k(wave * kPerWave + i, lane) >= k_left) voff[i] = kOutOfRange;
+    }
   }
 
   // Moves on to the next K-slice (a slice past the end of K reads all zeros).
-  __device__ __forceinline__ void advance() {
-    const uint64_t p = (((uint64_t)base_hi << 32) | base_lo) + (uint32_t)step;
-    base_lo = (uint32_t)p;
-    base_hi = (uint32_t)(p >> 32);
+  __device__ __forceinline__ void advance(int wave, int lane) {
+    // 48-bit base: the carry into bits 32..47 cannot reach the stride field
+    const uint64_t p = (((uint64_t)(uint32_t)rsrc[1] << 32) | (uint32_t)rsrc[0]) + (uint32_t)step;
+    rsrc[0] = (int)(uint32_t)p;
+    rsrc[1] = (int)(uint32_t)(p >> 32);
     remaining -= step;
+    rsrc[2] = max(remaining, 0);
     k_left -= BK;
+    mask_k_tail(wave, lane);
   }
 
-  // Group gi of this wave's copy instructions of the current slice into the
-  // tile at LDS byte address `tile_lds`.
+  // Copy instruction i of this wave for the current slice, into the tile at
+  // LDS byte address `tile_lds`.
   //
   // Written as inline assembly on purpose: the compiler then neither knows
   // that LDS is being written nor counts the loads in vmcnt, so it does not
   // put a full vmcnt(0) wait in front of every LDS read of the OTHER stages.
   // The kernel waits for a slice explicitly and publishes it with a barrier
   // before anyone reads it.
-  __device__ __forceinline__ void issue_group(int gi, uint32_t tile_lds, int wave) const {
-    i32x4_t rsrc;
-    rsrc[0] = (int)base_lo;
-    rsrc[1] = (int)(base_hi & 0xffffu);                       // stride 0
-    rsrc[2] = remaining > 0 ? remaining + kImmSpan : 0;       // num_records
-    rsrc[3] = kRsrcFlags;
-    uint32_t off[kGroup];
-#pragma unroll
-    for (int j = 0; j < kGroup; ++j) {
-      off[j] = voff[gi * kGroup + j];
-      if (KC) off[j] = kpack[gi * kGroup + j] < k_left ? off[j] : kOutOfRange;  // K tail
-    }
-    const uint32_t dst = tile_lds + (uint32_t)(wave * kPerWave + gi * kGroup) * 1024u;
-    if constexpr (kGroup == 4) {
-      asm volatile(
-          "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-          "buffer_load_dwordx4 %1, %5, 0 offen lds\n\t"
-          "buffer_load_dwordx4 %2, %5, 0 offen offset:1024 lds\n\t"
-          "buffer_load_dwordx4 %3, %5, 0 offen offset:2048 lds\n\t"
-          "buffer_load_dwordx4 %4, %5, 0 offen offset:3072 lds"
-          :: "s"(dst), "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "s"(rsrc)
-          : "memory", "m0");
-    } else if constexpr (kGroup == 2) {
-      asm volatile(
-          "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-          "buffer_load_dwordx4 %1, %3, 0 offen lds\n\t"
-          "buffer_load_dwordx4 %2, %3, 0 offen offset:1024 lds"
-          :: "s"(dst), "v"(off[0]), "v"(off[1]), "s"(rsrc) : "memory", "m0");
-    } else {
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                   :: "s"(dst), "v"(off[0]), "s"(rsrc) : "memory", "m0");
-    }
+  __device__ __forceinline__ void issue(int i, uint32_t tile_lds, int wave) const {
+    const uint32_t dst = tile_lds + (uint32_t)(wave * kPerWave + i) * 1024u;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(dst), "v"(voff[i]), "s"(rsrc) : "memory", "m0");
   }
 
   // MFMA fragment of the 32-row sub-tile starting at `row32`, K step `kk`
@@ -242,14 +228,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, int
   constexpr bool B_KC = MODE == GEMM_FWD;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % 16 == 0, "tile shape");
-  static_assert(NS >= 4 && NS <= 6, "LDS stages");
+  static_assert((NS >= 4 && NS <= 6) || (NS == 2 && BK == 64), "LDS stages");
   using ATile = DmaTile<BM, BK, NW, A_KC>;
   using BTile = DmaTile<BN, BK, NW, B_KC>;
   constexpr int kStageBytes = ATile::kBytes + BTile::kBytes;
   constexpr int kStageElems = kStageBytes / 2;
   constexpr int kLoads = ATile::kPerWave + BTile::kPerWave;  // per wave per slice
-  constexpr int kGroups = ATile::kGroups + BTile::kGroups;   // asm groups per slice
-  static_assert(kLoads * (NS - 3) < 64, "vmcnt is a 6-bit counter");
+  static_assert(NS == 2 || kLoads * (NS - 3) < 64, "vmcnt is a 6-bit counter");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -290,10 +275,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, int
   ta.init(A_KC ? A + (int64_t)m0 * lda : A + m0, wave, lane, lda, m_valid, M - m0, K);
   tb.init(B_KC ? B + (int64_t)n0 * ldb : B + n0, wave, lane, ldb, n_valid, N - n0, K);
 
-  // gi-th copy group of the current slice (A tile's groups first)
-  auto issue_group = [&](int gi, uint32_t stage_lds) {
-    if (gi < ATile::kGroups) ta.issue_group(gi, stage_lds, wave);
-    else tb.issue_group(gi - ATile::kGroups, stage_lds + ATile::kBytes, wave);
+  // j-th copy instruction of this wave for the current slice (A tile's first)
+  auto issue_load = [&](int j, uint32_t stage_lds) {
+    if (j < ATile::kPerWave) ta.issue(j, stage_lds, wave);
+    else tb.issue(j - ATile::kPerWave, stage_lds + ATile::kBytes, wave);
   };
 
   // acc[i][j] holds the TRANSPOSE of the 32x32 block (i, j) of C: the MFMA is
@@ -307,82 +292,191 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, int
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // ---- software pipeline over the K-slices (NS LDS stages, NS >= 4)
-  //
-  // At the top of iteration kt: slices kt and kt+1 are visible to every wave,
-  // slice kt+2 is in flight, the MFMA fragments of (kt, K step 0) are already
-  // in registers, and the stage of slice kt-1 is free.  The iteration
-  //   * issues the copy of slice kt+NS-1 into that free stage, its groups of
-  //     copy instructions spread between the MFMAs,
-  //   * runs the MFMAs of slice kt, reading the fragments of the next K step
-  //     one LDS read behind each MFMA; the last K step prefetches the first
-  //     fragments of slice kt+1, so the MFMA pipe does not drain at the barrier,
-  //   * waits until its own share of slice kt+2 has landed and meets the other
-  //     waves at the barrier, which publishes slice kt+2 and frees stage kt.
-  // Slices past the end of K are zero-filled dummies; nothing is conditional.
   constexpr int KK = BK / 16;                    // MFMA K steps per slice
   constexpr int kMmaPerSlice = KK * TM * TN;
-  constexpr int kEvery = kMmaPerSlice / kGroups; // MFMAs between two copy groups
   static_assert(KK % 2 == 0, "fragment double buffer is indexed by the parity of the K step");
-  static_assert(kEvery >= 1 && TM + TN <= TM * TN, "interleaving plan");
-
+  static_assert(TM + TN <= TM * TN, "interleaving plan");
+  static_assert(NW == 4, "one copy of the K loop per wave");
   const int k_tiles = (K + BK - 1) / BK;
-#pragma unroll
-  for (int s = 0; s < NS - 1; ++s) {
-#pragma unroll
-    for (int gi = 0; gi < kGroups; ++gi) issue_group(gi, lds_base + s * kStageBytes);
-    ta.advance();
-    tb.advance();
-  }
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 3) * kLoads) : "memory");
-  __syncthreads();
-
   uint4 fa[2][TM], fb[2][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-    fa[0][i] = ATile::frag(smem, wave_m * (BM / WM) + i * 32, 0, lane);
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-    fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 32, 0, lane);
 
-  int stage = 0;
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int stage_next = stage + 1 == NS ? 0 : stage + 1;
-    const int stage_free = stage == 0 ? NS - 1 : stage - 1;
-    const uint32_t free_lds = lds_base + (uint32_t)stage_free * kStageBytes;
-    const uint16_t* la = smem + stage * kStageElems;
-    const uint16_t* lb = la + ATile::kBytes / 2;
-    const uint16_t* la_next = smem + stage_next * kStageElems;
-    const uint16_t* lb_next = la_next + ATile::kBytes / 2;
+  if constexpr (NS == 2) {
+    // ---- two stages of 64 values of K, one barrier per slice
+    //
+    // A [row][k] operand then moves whole 128-byte lines (half as many L2
+    // requests as 64-byte pieces of rows).  Iteration kt runs the four K steps
+    // of slice kt; the barrier sits in front of the LAST K step:
+    //   * K steps 0..2 read their fragments from slice kt's stage; by the
+    //     barrier every wave has read all of it, so the stage is free, and has
+    //     waited for its share of slice kt+1, so that slice is published;
+    //   * K step 3 prefetches the first fragments of slice kt+1 and starts the
+    //     copy of slice kt+2 into the freed stage; K step 0 of the next
+    //     iteration issues the second half of that copy.  The copy then has K
+    //     steps 1 and 2 (32 MFMAs) to land.
+    constexpr int kHalf = kLoads / 2;
+    static_assert(kLoads % 2 == 0, "the copy of a slice is issued in two halves");
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      const int cur = kk & 1;
-      const uint16_t* pa = kk + 1 < KK ? la : la_next;
-      const uint16_t* pb = kk + 1 < KK ? lb : lb_next;
-      const int kk_pre = kk + 1 < KK ? kk + 1 : 0;
+    for (int j = 0; j < kLoads; ++j) issue_load(j, lds_base);
+    ta.advance(wave, lane);
+    tb.advance(wave, lane);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
+    for (int j = 0; j < kHalf; ++j) issue_load(j, lds_base + kStageBytes);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kHalf) : "memory");
+    __syncthreads();
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          acc[i][j] = Mma<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
-          const int q = i * TN + j;
-          if (q < TM)
-            fa[cur ^ 1][q] = ATile::frag(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
-          else if (q < TM + TN)
-            fb[cur ^ 1][q - TM] =
-                BTile::frag(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
-          const int n = kk * TM * TN + q;
-          if (n % kEvery == kEvery / 2 && n / kEvery < kGroups)
-            issue_group(n / kEvery, free_lds);
-          __builtin_amdgcn_sched_barrier(0);
+    for (int i = 0; i < TM; ++i)
+      fa[0][i] = ATile::frag(smem, wave_m * (BM / WM) + i * 32, 0, lane);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 32, 0, lane);
+
+    auto k_loop = [&](auto phase_tag) {
+      constexpr int kPhase = decltype(phase_tag)::value;
+      constexpr int kPerStep = TM * TN;           // MFMAs per K step
+      for (int kt = 0; kt < k_tiles; ++kt) {
+        const int stage = kt & 1;
+        const uint32_t cur_lds = lds_base + (uint32_t)stage * kStageBytes;
+        const uint32_t other_lds = lds_base + (uint32_t)(stage ^ 1) * kStageBytes;
+        const uint16_t* la = smem + stage * kStageElems;
+        const uint16_t* lb = la + ATile::kBytes / 2;
+        const uint16_t* la_next = smem + (stage ^ 1) * kStageElems;
+        const uint16_t* lb_next = la_next + ATile::kBytes / 2;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          if (kk == KK - 1) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): my reads of this stage are done
+            __syncthreads();
+          }
+          const int cur = kk & 1;
+          const uint16_t* pa = kk + 1 < KK ? la : la_next;
+          const uint16_t* pb = kk + 1 < KK ? lb : lb_next;
+          const int kk_pre = kk + 1 < KK ? kk + 1 : 0;
+#pragma unroll
+          for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+              acc[i][j] = Mma<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
+              const int q = i * TN + j;
+              if (q < TM)
+                fa[cur ^ 1][q] = ATile::frag(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
+              else if (q < TM + TN)
+                fb[cur ^ 1][q - TM] =
+                    BTile::frag(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
+              // copy instruction c of a half sits behind MFMA
+              // (c * NW + phase) * kPerStep / (kHalf * NW) of its K step
+              if (kk == 0 || kk == KK - 1) {
+#pragma unroll
+                for (int c = 0; c < kHalf; ++c)
+                  if ((c * NW + kPhase) * kPerStep / (kHalf * NW) == q) {
+                    if (kk == 0) issue_load(kHalf + c, other_lds);  // rest of slice kt+1
+                    else issue_load(c, cur_lds);                    // start of slice kt+2
+                  }
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
+          if (kk == 0) {  // slice kt+1 is issued in full: move on to slice kt+2
+            ta.advance(wave, lane);
+            tb.advance(wave, lane);
+          }
         }
       }
+    };
+    switch (wave) {
+      case 0: k_loop(std::integral_constant<int, 0>{}); break;
+      case 1: k_loop(std::integral_constant<int, 1>{}); break;
+      case 2: k_loop(std::integral_constant<int, 2>{}); break;
+      default: k_loop(std::integral_constant<int, 3>{}); break;
     }
-    ta.advance();
-    tb.advance();
+  } else {
+    // ---- software pipeline over the K-slices (NS LDS stages, NS >= 4)
+    //
+    // At the top of iteration kt: slices kt and kt+1 are visible to every wave,
+    // slice kt+2 is in flight, the MFMA fragments of (kt, K step 0) are already
+    // in registers, and the stage of slice kt-1 is free.  The iteration
+    //   * issues the copy of slice kt+NS-1 into that free stage, one copy
+    //     instruction at a time between the MFMAs,
+    //   * runs the MFMAs of slice kt, reading the fragments of the next K step
+    //     one LDS read behind each MFMA; the last K step prefetches the first
+    //     fragments of slice kt+1, so the MFMA pipe does not drain at the barrier,
+    //   * waits until its own share of slice kt+2 has landed and meets the other
+    //     waves at the barrier, which publishes slice kt+2 and frees stage kt.
+    // Slices past the end of K are zero-filled dummies; nothing is conditional.
+    //
+    // The barrier releases the waves of a block together, and a copy instruction
+    // keeps the CU's one address unit busy for some 16 cycles: if every wave put
+    // its copies behind the same MFMAs, each would queue behind the others and
+    // hold up its own MFMAs.  The loop therefore exists once per wave (`phase`),
+    // with the copy instructions of wave w behind MFMAs that no other wave uses.
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s) {
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) issue_load(j, lds_base + s * kStageBytes);
+      ta.advance(wave, lane);
+      tb.advance(wave, lane);
+    }
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 3) * kLoads) : "memory");
     __syncthreads();
-    stage = stage_next;
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      fa[0][i] = ATile::frag(smem, wave_m * (BM / WM) + i * 32, 0, lane);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 32, 0, lane);
+
+    auto k_loop = [&](auto phase_tag) {
+      constexpr int kPhase = decltype(phase_tag)::value;
+      int stage = 0;
+      for (int kt = 0; kt < k_tiles; ++kt) {
+        const int stage_next = stage + 1 == NS ? 0 : stage + 1;
+        const int stage_free = stage == 0 ? NS - 1 : stage - 1;
+        const uint32_t free_lds = lds_base + (uint32_t)stage_free * kStageBytes;
+        const uint16_t* la = smem + stage * kStageElems;
+        const uint16_t* lb = la + ATile::kBytes / 2;
+        const uint16_t* la_next = smem + stage_next * kStageElems;
+        const uint16_t* lb_next = la_next + ATile::kBytes / 2;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          const int cur = kk & 1;
+          const uint16_t* pa = kk + 1 < KK ? la : la_next;
+          const uint16_t* pb = kk + 1 < KK ? lb : lb_next;
+          const int kk_pre = kk + 1 < KK ? kk + 1 : 0;
+#pragma unroll
+          for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+              acc[i][j] = Mma<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
+              const int q = i * TN + j;
+              if (q < TM)
+                fa[cur ^ 1][q] = ATile::frag(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
+              else if (q < TM + TN)
+                fb[cur ^ 1][q - TM] =
+                    BTile::frag(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
+              // copy instruction c of phase p sits behind MFMA
+              // (c * NW + p) * kMmaPerSlice / (kLoads * NW)
+              const int n = kk * TM * TN + q;
+#pragma unroll
+              for (int c = 0; c < kLoads; ++c)
+                if ((c * NW + kPhase) * kMmaPerSlice / (kLoads * NW) == n) issue_load(c, free_lds);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          }
+        }
+        ta.advance(wave, lane);
+        tb.advance(wave, lane);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 3) * kLoads) : "memory");
+        __syncthreads();
+        stage = stage_next;
+      }
+    };
+    switch (wave) {
+      case 0: k_loop(std::integral_constant<int, 0>{}); break;
+      case 1: k_loop(std::integral_constant<int, 1>{}); break;
+      case 2: k_loop(std::integral_constant<int, 2>{}); break;
+      default: k_loop(std::integral_constant<int, 3>{}); break;
+    }
   }
   // The zero-filled dummy slices are still landing in LDS: let them finish,
   // then the whole LDS allocation is free to stage the output tile.
@@ -699,12 +793,12 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
 // take a block at a time (256 CUs; live tiles come first in launch order, so a
 // round is really 256 wide), a tile costs a fixed prologue/epilogue
 // plus a per-K-slice time that depends on its shape (measured microseconds).
-// The shape with the least estimated time wins; `g.tile` (1..3) overrides the
-// choice for tuning.  Ragged experts add at most one partial tile each, which
+// The shape with the least estimated time wins; `g.tile` overrides the choice
+// for tuning (1..3 = the three shapes, 4 = 256x256 with two stages of 64).  Ragged experts add at most one partial tile each, which
 // the estimate ignores.
 template <int MODE>
 static int pick_tile(const GemmArgs& g) {
-  if (g.tile >= 1 && g.tile <= 3) return g.tile;
+  if (g.tile >= 1 && g.tile <= 4) return g.tile;
   const int64_t N = MODE == GEMM_FWD ? g.out_feat : g.in_feat;
   const int64_t K = MODE == GEMM_WGRAD ? g.n_rows / g.n_expert
                                        : (MODE == GEMM_FWD ? g.in_feat : g.out_feat);
@@ -724,8 +818,14 @@ static int pick_tile(const GemmArgs& g) {
 template <typename T, int MODE>
 static int launch_mode(const GemmArgs& g, hipStream_t s) {
   switch (pick_tile<MODE>(g)) {
-    case 1: return launch_cfg<T, 256, 256, 32, 2, 2, 4, MODE>(g, s);
+    case 1:
+      // Both FWD operands are [row][k] in memory: K slices of 64 move whole
+      // 128-byte lines and measured 7-8% faster there; the products with a
+      // [k][row] operand do as well or better with four stages of 32.
+      if (MODE == GEMM_FWD) return launch_cfg<T, 256, 256, 64, 2, 2, 2, MODE>(g, s);
+      return launch_cfg<T, 256, 256, 32, 2, 2, 4, MODE>(g, s);
     case 2: return launch_cfg<T, 128, 256, 32, 2, 2, 4, MODE>(g, s);
+    case 4: return launch_cfg<T, 256, 256, 64, 2, 2, 2, MODE>(g, s);
     default: return launch_cfg<T, 128, 128, 32, 2, 2, 4, MODE>(g, s);
   }
 }
