@@ -51,6 +51,15 @@ CONFIGS = {
 DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 PEAK = {"hbm": 8.0e12, "bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 
+# HBM bytes per launch (read + write) from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# counter runs of this script, scaled by what the same counters read for the
+# row-scatter kernel, whose traffic is known (factors 1.035 and 1.000).  Only
+# the workloads that were measured have an entry.
+MEASURED_TRAFFIC = {
+    ("cfg2", "grouped_linear_bwd"): (274.2 + 208.0) * 2 ** 20,
+    ("cfg2", "grouped_linear_fwd"): (153.7 + 80.0) * 2 ** 20,
+}
+
 
 def make_routing(cfg: dict, seed: int = 0):
     """(logits [T, E] float32 or None, idx [T, k] int64 or None): the seeded
@@ -285,7 +294,8 @@ def main():
         roofline = {"kernel": dom, "bound": "hbm", "achieved": round(amount / avg_s / 1e9, 2),
                     "peak": PEAK["hbm"] / 1e9, "unit": "GB/s"}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
-    roofline["traffic"] = None
+    traffic = MEASURED_TRAFFIC.get((args.config, dom))
+    roofline["traffic"] = None if traffic is None else round(traffic)
     roofline["avg_launch_us"] = kernels[dom]["avg_us"]
 
     result = {
