@@ -165,26 +165,21 @@ __global__ __launch_bounds__(kRouteThreads) void route_place_kernel(
   __syncthreads();
 
   const uint64_t lt_mask = ((uint64_t)1 << lane) - 1;
+  const int key_bits = 32 - __clz(max(n_expert - 1, 1));
 #pragma unroll
   for (int s = 0; s < kRowsPerWave; ++s) {
     const int64_t i = base + (int64_t)(w * kRowsPerWave + s) * kWave + lane;
     const int32_t key = keys[s];
     const bool valid = key >= 0;
-    int rank = 0, cnt = 0;
-    bool first = false;
-    uint64_t todo = __ballot(valid);
-    while (todo) {
-      const int leader = __ffsll((unsigned long long)todo) - 1;
-      const int32_t k0 = __shfl(key, leader, kWave);
-      const bool same = valid && key == k0;
-      const uint64_t m = __ballot(same);
-      if (same) {
-        rank = __popcll(m & lt_mask);
-        cnt = __popcll(m);
-        first = lane == leader;
-      }
-      todo &= ~m;
+    // lanes of this row with the same key: one ballot per bit of the key
+    uint64_t same = __ballot(valid);
+    for (int bit = 0; bit < key_bits; ++bit) {
+      const uint64_t vote = __ballot(valid && ((key >> bit) & 1));
+      same &= ((key >> bit) & 1) ? vote : ~vote;
     }
+    const int rank = __popcll(same & lt_mask);
+    const int cnt = __popcll(same);
+    const bool first = valid && (same & lt_mask) == 0;
     int32_t p = 0;
     if (valid) p = wave_cnt[w * n_expert + key] + rank;
     // every lane of the wave has read its counter before the leader of each
