@@ -14,6 +14,7 @@ namespace fmoe {
 
 constexpr int kDispThreads = 256;
 constexpr int kDispWaves = kDispThreads / kWave;
+constexpr int kCombineUnroll = 4;   // 16-byte packs a lane of the combine kernels has in flight
 constexpr int kMaxGrid = 256 * 32;  // enough resident waves for 256 CUs
 
 __device__ __forceinline__ int64_t live_rows(int64_t n_rows,
@@ -146,24 +147,42 @@ __global__ __launch_bounds__(kDispThreads) void combine_fwd_kernel(
       my_r = inv[t * top_k + lane];
       my_s = score ? Elem<T>::to_acc(score[t * top_k + lane]) : (acc_t)1;
     }
-    for (int64_t c = lane; c < row_vecs; c += kWave) {
-      acc_t acc[VEC];
+    // kCombineUnroll packs per lane per step: all their loads are issued
+    // before the first is used
+    for (int64_t c0 = lane; c0 < row_vecs; c0 += kWave * kCombineUnroll) {
+      acc_t acc[kCombineUnroll][VEC];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) acc[v] = 0;
+      for (int u = 0; u < kCombineUnroll; ++u)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[u][v] = 0;
       for (int j = 0; j < top_k; ++j) {
         // lanes beyond the row's last pack are not in this loop, so a
         // shuffle could not read them; lane_value can
         const int32_t r = lane_value(my_r, j);
         const acc_t s = lane_value(my_s, j);
         if (r < 0) continue;
-        const Pk p = *reinterpret_cast<const Pk*>(buf + (int64_t)r * d + c * VEC);
+        const T* src = buf + (int64_t)r * d;
+        Pk p[kCombineUnroll];
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) acc[v] += s * Elem<T>::to_acc(p.v[v]);
+        for (int u = 0; u < kCombineUnroll; ++u) {
+          const int64_t c = c0 + (int64_t)u * kWave;
+          if (c < row_vecs) p[u] = *reinterpret_cast<const Pk*>(src + c * VEC);
+        }
+#pragma unroll
+        for (int u = 0; u < kCombineUnroll; ++u)
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) acc[u][v] += s * Elem<T>::to_acc(p[u].v[v]);
       }
-      Pk o;
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) o.v[v] = Elem<T>::from_acc(acc[v]);
-      *reinterpret_cast<Pk*>(y + t * d + c * VEC) = o;
+      for (int u = 0; u < kCombineUnroll; ++u) {
+        const int64_t c = c0 + (int64_t)u * kWave;
+        if (c < row_vecs) {
+          Pk o;
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) o.v[v] = Elem<T>::from_acc(acc[u][v]);
+          *reinterpret_cast<Pk*>(y + t * d + c * VEC) = o;
+        }
+      }
     }
   }
 }
@@ -193,17 +212,30 @@ __global__ __launch_bounds__(kDispThreads) void combine_bwd_kernel(
       const acc_t s = lane_value(my_s, j);
       acc_t dot = 0;
       if (r >= 0) {
-        for (int64_t c = lane; c < row_vecs; c += kWave) {
-          const Pk g = *reinterpret_cast<const Pk*>(dy + t * d + c * VEC);
-          const Pk o = *reinterpret_cast<const Pk*>(buf + (int64_t)r * d + c * VEC);
-          Pk w;
+        for (int64_t c0 = lane; c0 < row_vecs; c0 += kWave * kCombineUnroll) {
+          Pk g[kCombineUnroll], o[kCombineUnroll];
 #pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            const acc_t gv = Elem<T>::to_acc(g.v[v]);
-            dot += gv * Elem<T>::to_acc(o.v[v]);
-            w.v[v] = Elem<T>::from_acc(s * gv);
+          for (int u = 0; u < kCombineUnroll; ++u) {
+            const int64_t c = c0 + (int64_t)u * kWave;
+            if (c < row_vecs) {
+              g[u] = *reinterpret_cast<const Pk*>(dy + t * d + c * VEC);
+              o[u] = *reinterpret_cast<const Pk*>(buf + (int64_t)r * d + c * VEC);
+            }
           }
-          *reinterpret_cast<Pk*>(dbuf + (int64_t)r * d + c * VEC) = w;
+#pragma unroll
+          for (int u = 0; u < kCombineUnroll; ++u) {
+            const int64_t c = c0 + (int64_t)u * kWave;
+            if (c < row_vecs) {
+              Pk w;
+#pragma unroll
+              for (int v = 0; v < VEC; ++v) {
+                const acc_t gv = Elem<T>::to_acc(g[u].v[v]);
+                dot += gv * Elem<T>::to_acc(o[u].v[v]);
+                w.v[v] = Elem<T>::from_acc(s * gv);
+              }
+              *reinterpret_cast<Pk*>(dbuf + (int64_t)r * d + c * VEC) = w;
+            }
+          }
         }
 #pragma unroll
         for (int off = kWave / 2; off > 0; off >>= 1)
