@@ -530,8 +530,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, int
   }
 }
 
-// Rows per remainder tile (see the kernel below).
+// Remainder tiles (see the kernels below): 64 rows, K slices of 32 in 6 LDS
+// stages.  A slice of such a tile is a quarter of the MFMA work of a 256-row
+// one, so its copies need more slices of lead to cover the memory latency.
 constexpr int kSmallRows = 64;
+constexpr int kSmallBK = 32;
+constexpr int kSmallStages = 6;
 
 // Whether tile shape BM x BN (4 waves) has a remainder shape kSmallRows x BN
 // (the 4 waves side by side) that the pipeline's interleaving plan accepts.
@@ -687,7 +691,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   __syncthreads();
   if constexpr (kSmall) {
     if (small) {
-      gemm_tile<T, kSmallRows, BN, BK, 1, NW, NS, MODE>(g, smem, s_expert, s_row, n_tile);
+      gemm_tile<T, kSmallRows, BN, kSmallBK, 1, NW, kSmallStages, MODE>(g, smem, s_expert, s_row,
+                                                                       n_tile);
       return;
     }
   }
@@ -738,7 +743,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
   __syncthreads();
   if constexpr (kSmall) {
     if (small) {
-      gemm_tile<T, kSmallRows, BN, BK, 1, NW, NS, GEMM_DGRAD>(gd, smem, s_expert, s_row, n_tile);
+      gemm_tile<T, kSmallRows, BN, kSmallBK, 1, NW, kSmallStages, GEMM_DGRAD>(gd, smem, s_expert,
+                                                                             s_row, n_tile);
       return;
     }
   }
@@ -754,7 +760,10 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   using BTile = DmaTile<BN, BK, NW, MODE == GEMM_FWD>;
   constexpr size_t pipe_bytes = NS * (ATile::kBytes + BTile::kBytes);
   constexpr size_t out_bytes = (size_t)BM * (BN + 8) * 2;   // staged output tile
-  constexpr size_t lds_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
+  constexpr size_t small_bytes = has_small_tiles<BM, BN, MODE>()
+      ? (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2 : 0;
+  constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
+  constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
   auto kern = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, NS, MODE>;
   static bool configured = false;  // attribute is per function, set once
@@ -850,7 +859,9 @@ static int launch_bwd_t(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
   constexpr int BM = 256, BN = 256, BK = 32, WM = 2, WN = 2, NS = 4, NT = WM * WN * 64;
   constexpr size_t pipe_bytes = (size_t)NS * (BM + BN) * BK * 2;
   constexpr size_t out_bytes = (size_t)BM * (BN + 8) * 2;
-  constexpr size_t lds_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
+  constexpr size_t small_bytes = (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2;
+  constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
+  constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
   auto kern = gemm_bwd_kernel<T, BM, BN, BK, WM, WN, NS>;
   static bool configured = false;  // attribute is per function, set once
