@@ -9,9 +9,10 @@
 namespace fmoe {
 
 static thread_local char g_err[512] = "";
-static int g_gemm_path = 0;  // 0 = automatic, 1 = scalar kernel only
+static int g_gemm_path = 0;  // 0 = automatic, 1 = scalar kernel only (2..5 set g_tile instead)
 // tuning aid: FMOE_GEMM_TILE=1..4 forces one MFMA tile configuration (0 / unset = automatic)
-static int g_tile = getenv("FMOE_GEMM_TILE") ? atoi(getenv("FMOE_GEMM_TILE")) : 0;
+static const int g_env_tile = getenv("FMOE_GEMM_TILE") ? atoi(getenv("FMOE_GEMM_TILE")) : 0;
+static int g_tile = g_env_tile;
 
 int set_error(int code, const char* fmt, ...) {
   va_list ap;
@@ -126,8 +127,10 @@ extern "C" const char* fmoe_version(void) { return "fastmoe_amd 0.1 (gfx950)"; }
 extern "C" const char* fmoe_last_error(void) { return g_err; }
 
 extern "C" int fmoe_set_gemm_path(int path) {
-  FMOE_REQUIRE(path == 0 || path == 1, FMOE_ERR_INVALID, "gemm path must be 0 or 1");
-  g_gemm_path = path;
+  FMOE_REQUIRE(path >= 0 && path <= 5, FMOE_ERR_INVALID, "gemm path must be 0..5");
+  // 2..5: matrix-core kernel with tile configuration 1..4 forced (tests, tuning)
+  g_gemm_path = path == 1 ? 1 : 0;
+  g_tile = path >= 2 ? path - 1 : g_env_tile;
   return FMOE_OK;
 }
 

@@ -420,5 +420,7 @@ def scatter_reduce(dbuf: torch.Tensor, inv: torch.Tensor, n_tokens: int,
 
 
 def set_gemm_path(path: int) -> None:
-    """0 = matrix-core kernel where the shape allows, 1 = scalar kernel only."""
+    """0 = matrix-core kernel where the shape allows (tile shape chosen by the
+    library), 1 = scalar kernel only, 2..5 = matrix-core kernel with tile
+    configuration 1..4 forced (for tests and tuning)."""
     _lib.check(_L.fmoe_set_gemm_path(path), "set_gemm_path")

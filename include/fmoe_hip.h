@@ -227,7 +227,10 @@ int fmoe_seg_off_from_host_counts(const int64_t* expert_count_host,
 
 /*
  * Selects the grouped-GEMM kernel family for bf16/f16: 0 = automatic (MFMA
- * where the shape allows), 1 = force the scalar kernel (testing aid).
+ * where the shape allows, tile shape from the library's cost model), 1 = force
+ * the scalar kernel, 2..5 = MFMA with tile configuration 1..4 forced (256x256,
+ * 128x256, 128x128, 256x256 with K slices of 64).  A testing and tuning aid
+ * with no counterpart in the reference; process-wide, not thread-safe.
  */
 int fmoe_set_gemm_path(int path);
 

@@ -70,9 +70,26 @@ def test_matrix_core_kernel(dt, with_bias, counts, in_f, out_f):
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
 def test_matrix_core_large_tiles_and_dead_rows(dt):
-    # average rows per expert >= 768 selects the 256x256 tiles; 37 rows past
+    # a mid-size problem with the tile shape left to the library; 37 rows past
     # seg_off[E] are dead and must not be read as part of any expert
     _run([1000, 0, 1531, 800], 512, 1024, DTYPES[dt], True, path=0, extra_rows=37)
+
+
+# every tile configuration of the matrix-core kernel, forced, on shapes with
+# partial tiles in M, N and K, remainders of every length class (none, up to 64,
+# up to 128, above half a tile), empty experts and dead rows at the end
+FORCED = [
+    ([300, 0, 257, 64, 1, 200, 513], 136, 264),
+    ([1024 + 17, 1024 - 9, 0, 130], 72, 520),
+    ([255, 129, 128, 65, 63], 264, 256),
+]
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4])
+@pytest.mark.parametrize("counts,in_f,out_f", FORCED)
+def test_matrix_core_forced_tile(dt, tile, counts, in_f, out_f):
+    _run(counts, in_f, out_f, DTYPES[dt], True, path=1 + tile, extra_rows=5)
 
 
 @pytest.mark.parametrize("n_expert", [257, 600, 4096])
