@@ -217,10 +217,19 @@ __device__ __forceinline__ void tile_order(int t, int rows, int cols, int& row, 
   col = blk * 8 + r / patch_rows;
 }
 
+// Where a tile sits in the rows of its expert.
+struct TileRows {
+  int e;        // expert
+  int m0;       // first row of the tile inside the expert
+  int row0;     // first row of the expert
+  int cnt;      // rows of the expert
+};
+
 // One output tile: rows [m0, m0 + BM) of expert e's row range (WGRAD: of its
-// out_feat x in_feat gradient) by columns [n_tile * BN, + BN).
+// out_feat x in_feat gradient) by columns [n_tile * BN, + BN); `where` names
+// the expert, m0 and the expert's rows.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
-__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, int e, int m0,
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
                                           int n_tile) {
   constexpr int NW = WM * WN;
   constexpr int NT = NW * 64;
@@ -241,9 +250,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, int
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave / WN, wave_n = wave % WN;
   const int in_f = g.in_feat, out_f = g.out_feat;
-  e = __builtin_amdgcn_readfirstlane(e);
-  const int row0 = __builtin_amdgcn_readfirstlane(g.seg_off[e]);
-  const int cnt = __builtin_amdgcn_readfirstlane(g.seg_off[e + 1]) - row0;
+  const int e = __builtin_amdgcn_readfirstlane(where.e);
+  const int row0 = __builtin_amdgcn_readfirstlane(where.row0);
+  const int cnt = __builtin_amdgcn_readfirstlane(where.cnt);
 
   int M, N, K, lda, ldb, ldc;
   const uint16_t *A, *B;
@@ -264,7 +273,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, int
     B = (const uint16_t*)g.b + (int64_t)row0 * in_f;        ldb = in_f;
     C = (T*)g.c + (int64_t)e * out_f * in_f;                ldc = in_f;
   }
-  m0 = __builtin_amdgcn_readfirstlane(m0);
+  const int m0 = __builtin_amdgcn_readfirstlane(where.m0);
   const int n0 = __builtin_amdgcn_readfirstlane(n_tile) * BN;
   if (m0 >= M || n0 >= N) return;
   const int m_valid = min(BM, M - m0), n_valid = min(BN, N - n0);
@@ -580,29 +589,47 @@ __device__ __forceinline__ int tile_number(int pid, int live) {
 }
 
 // Row tiles of a ragged product.  The BM-row tiles of all experts are numbered
-// first, one expert after the other, the remainder tiles behind them.  Each
-// thread cuts the rows of a contiguous run of experts and a block-wide scan
-// turns the sums into first-tile numbers; the thread whose run contains a
-// given row tile walks the run to find its owner.
+// first, one expert after the other, the remainder tiles behind them.
+//
+// Up to 64 experts: lane x of EVERY wave cuts the rows of expert x and a wave
+// scan turns the counts into first-tile numbers, so no LDS and no barrier are
+// involved and the owner of a tile is read from its lane.  More experts: each
+// thread cuts the rows of a contiguous run of experts, the scan runs over the
+// whole block through LDS, and the thread whose run contains a given row tile
+// walks the run to find its owner.
 template <int BM, bool SMALL, int NW>
 struct RowTiles {
+  bool by_lane;            // the up-to-64-experts scheme
   int x_lo, x_hi;          // this thread's run of experts
   int mine_f, mine_s;      // BM-row / remainder tiles in the run
   int first_f, first_s;    // number of the run's first tile of either kind
   int rows_f, rows_s;      // totals over all experts
+  int my_row0, my_cnt;     // by_lane: the expert of this lane
 
-  // Contains a __syncthreads(); s_wave_sum has 2 * NW entries.
+  // May contain a __syncthreads(); s_wave_sum has 2 * NW entries.
   __device__ __forceinline__ void scan(const int32_t* seg_off, int n_expert, int* s_wave_sum) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int per_thread = (n_expert + NW * 64 - 1) / (NW * 64);
-    x_lo = min(tid * per_thread, n_expert);
-    x_hi = min(x_lo + per_thread, n_expert);
+    by_lane = n_expert <= 64;
     mine_f = mine_s = 0;
-    for (int x = x_lo; x < x_hi; ++x) {
-      int f, sm;
-      cut_rows<BM, SMALL>(seg_off[x + 1] - seg_off[x], f, sm);
-      mine_f += f;
-      mine_s += sm;
+    if (by_lane) {
+      x_lo = lane;
+      x_hi = lane < n_expert ? lane + 1 : lane;
+      my_row0 = my_cnt = 0;
+      if (lane < n_expert) {
+        my_row0 = seg_off[lane];
+        my_cnt = seg_off[lane + 1] - my_row0;
+        cut_rows<BM, SMALL>(my_cnt, mine_f, mine_s);
+      }
+    } else {
+      const int per_thread = (n_expert + NW * 64 - 1) / (NW * 64);
+      x_lo = min(tid * per_thread, n_expert);
+      x_hi = min(x_lo + per_thread, n_expert);
+      for (int x = x_lo; x < x_hi; ++x) {
+        int f, sm;
+        cut_rows<BM, SMALL>(seg_off[x + 1] - seg_off[x], f, sm);
+        mine_f += f;
+        mine_s += sm;
+      }
     }
     int incl_f = mine_f, incl_s = mine_s;  // inclusive scans inside the wave
 #pragma unroll
@@ -614,13 +641,18 @@ struct RowTiles {
         if (lane >= d) incl_s += up_s;
       }
     }
+    first_f = incl_f - mine_f;
+    first_s = incl_s - mine_s;
+    if (by_lane) {
+      rows_f = __builtin_amdgcn_readlane(incl_f, 63);
+      rows_s = __builtin_amdgcn_readlane(incl_s, 63);
+      return;
+    }
     if (lane == 63) {
       s_wave_sum[wave] = incl_f;
       s_wave_sum[NW + wave] = incl_s;
     }
     __syncthreads();
-    first_f = incl_f - mine_f;
-    first_s = incl_s - mine_s;
     rows_f = rows_s = 0;
 #pragma unroll
     for (int w2 = 0; w2 < NW; ++w2) {
@@ -634,24 +666,46 @@ struct RowTiles {
     }
   }
 
-  // The owner of row tile v (of the remainder kind if `small`) stores the
-  // expert and the tile's first row inside the expert; the caller then syncs.
-  __device__ __forceinline__ void find(const int32_t* seg_off, int v, bool small,
-                                       int* s_expert, int* s_row) const {
+  // Owner of row tile v (of the remainder kind if `small`), v below the total
+  // of its kind.  s_out has 4 entries; may contain a __syncthreads().
+  __device__ __forceinline__ TileRows find(const int32_t* seg_off, int v, bool small,
+                                           int* s_out) const {
     const int first = small ? first_s : first_f, mine = small ? mine_s : mine_f;
-    if (v < first || v >= first + mine) return;
-    int at = first;
-    for (int x = x_lo; x < x_hi; ++x) {
-      int f, sm;
-      cut_rows<BM, SMALL>(seg_off[x + 1] - seg_off[x], f, sm);
-      const int tx = small ? sm : f;
-      if (v < at + tx) {
-        *s_expert = x;
-        *s_row = small ? f * BM + (v - at) * kSmallRows : (v - at) * BM;
-        return;
-      }
-      at += tx;
+    const bool own = v >= first && v < first + mine;
+    TileRows t;
+    if (by_lane) {
+      const int owner = __ffsll((unsigned long long)__ballot(own)) - 1;  // exactly one lane
+      const int at = __builtin_amdgcn_readlane(first, owner);
+      const int f = __builtin_amdgcn_readlane(mine_f, owner);
+      t.e = owner;
+      t.m0 = small ? f * BM + (v - at) * kSmallRows : (v - at) * BM;
+      t.row0 = __builtin_amdgcn_readlane(my_row0, owner);
+      t.cnt = __builtin_amdgcn_readlane(my_cnt, owner);
+      return t;
     }
+    if (own) {
+      int at = first;
+      for (int x = x_lo; x < x_hi; ++x) {
+        const int r0 = seg_off[x], c = seg_off[x + 1] - r0;
+        int f, sm;
+        cut_rows<BM, SMALL>(c, f, sm);
+        const int tx = small ? sm : f;
+        if (v < at + tx) {
+          s_out[0] = x;
+          s_out[1] = small ? f * BM + (v - at) * kSmallRows : (v - at) * BM;
+          s_out[2] = r0;
+          s_out[3] = c;
+          break;
+        }
+        at += tx;
+      }
+    }
+    __syncthreads();
+    t.e = s_out[0];
+    t.m0 = s_out[1];
+    t.row0 = s_out[2];
+    t.cnt = s_out[3];
+    return t;
   }
 };
 
@@ -664,7 +718,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   constexpr bool kSmall = has_small_tiles<BM, BN, MODE>();
   static_assert(!kSmall || NW == 4, "remainder tiles put 4 waves side by side");
   extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];  // [stage][A | B]
-  __shared__ int s_expert, s_row, s_wave_sum[2 * NW];
+  __shared__ int s_owner[4], s_wave_sum[2 * NW];
 
   const int pid = blockIdx.x;
   if (MODE == GEMM_WGRAD) {
@@ -673,7 +727,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
     if (t >= live) return;
     int m_tile, n_tile;
     tile_order(t % (tiles_n * tiles_m), tiles_m, tiles_n, m_tile, n_tile);
-    gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, t / (tiles_n * tiles_m), m_tile * BM,
+    const int e = t / (tiles_n * tiles_m);
+    const int row0 = g.seg_off[e];
+    gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, {e, m_tile * BM, row0, g.seg_off[e + 1] - row0},
                                                 n_tile);
     return;
   }
@@ -687,16 +743,14 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   int v, n_tile;
   if (small) tile_order(t - live_f, rows.rows_s, tiles_n, v, n_tile);
   else tile_order(t, rows.rows_f, tiles_n, v, n_tile);
-  rows.find(g.seg_off, v, small, &s_expert, &s_row);
-  __syncthreads();
+  const TileRows where = rows.find(g.seg_off, v, small, s_owner);
   if constexpr (kSmall) {
     if (small) {
-      gemm_tile<T, kSmallRows, BN, kSmallBK, 1, NW, kSmallStages, MODE>(g, smem, s_expert, s_row,
-                                                                       n_tile);
+      gemm_tile<T, kSmallRows, BN, kSmallBK, 1, NW, kSmallStages, MODE>(g, smem, where, n_tile);
       return;
     }
   }
-  gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, s_expert, s_row, n_tile);
+  gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, where, n_tile);
 }
 
 // Both gradient products of one grouped linear in one launch: the BM-row
@@ -713,7 +767,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
   constexpr bool kSmall = has_small_tiles<BM, BN, GEMM_DGRAD>();
   static_assert(!kSmall || NW == 4, "remainder tiles put 4 waves side by side");
   extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];
-  __shared__ int s_expert, s_row, s_wave_sum[2 * NW];
+  __shared__ int s_owner[4], s_wave_sum[2 * NW];
 
   RowTiles<BM, kSmall, NW> rows;
   rows.scan(gd.seg_off, gd.n_expert, s_wave_sum);
@@ -731,24 +785,25 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
     const int tw = t - w_begin;
     int m_tile, n_tile;
     tile_order(tw % per_expert_w, tiles_m_w, tiles_n_w, m_tile, n_tile);
-    gemm_tile<T, BM, BN, BK, WM, WN, NS, GEMM_WGRAD>(gw, smem, tw / per_expert_w, m_tile * BM,
-                                                      n_tile);
+    const int e = tw / per_expert_w;
+    const int row0 = gw.seg_off[e];
+    gemm_tile<T, BM, BN, BK, WM, WN, NS, GEMM_WGRAD>(
+        gw, smem, {e, m_tile * BM, row0, gw.seg_off[e + 1] - row0}, n_tile);
     return;
   }
   const bool small = t >= live_d;
   int v, n_tile;
   if (small) tile_order(t - s_begin, rows.rows_s, tiles_n_d, v, n_tile);
   else tile_order(t, rows.rows_f, tiles_n_d, v, n_tile);
-  rows.find(gd.seg_off, v, small, &s_expert, &s_row);
-  __syncthreads();
+  const TileRows where = rows.find(gd.seg_off, v, small, s_owner);
   if constexpr (kSmall) {
     if (small) {
-      gemm_tile<T, kSmallRows, BN, kSmallBK, 1, NW, kSmallStages, GEMM_DGRAD>(gd, smem, s_expert,
-                                                                             s_row, n_tile);
+      gemm_tile<T, kSmallRows, BN, kSmallBK, 1, NW, kSmallStages, GEMM_DGRAD>(gd, smem, where,
+                                                                             n_tile);
       return;
     }
   }
-  gemm_tile<T, BM, BN, BK, WM, WN, NS, GEMM_DGRAD>(gd, smem, s_expert, s_row, n_tile);
+  gemm_tile<T, BM, BN, BK, WM, WN, NS, GEMM_DGRAD>(gd, smem, where, n_tile);
 }
 
 // ------------------------------------------------------------------ host side
