@@ -525,17 +525,33 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, Til
     }
   }
   __syncthreads();
+  // every thread moves one fixed 16-byte column pack of every kRowsPerStep-th row
   constexpr int kRowPacks = BN / 8;                  // 16-byte packs per tile row
-  constexpr int kPacksPerThread = BM * kRowPacks / NT;
-  static_assert((BM * kRowPacks) % NT == 0, "output tile must split evenly over the threads");
-#pragma unroll 4
-  for (int it = 0; it < kPacksPerThread; ++it) {
-    const int c = tid + it * NT;
-    const int row = c / kRowPacks, pk = c % kRowPacks;
-    const int m = m0 + row, n = n0 + pk * 8;
-    if (m < M && n < N)   // N is a multiple of 8: a pack is all in or all out
-      *reinterpret_cast<uint4*>(C + (int64_t)m * ldc + n) =
-          *reinterpret_cast<const uint4*>(stage_c + row * kLdc + pk * 8);
+  constexpr int kRowsPerStep = NT / kRowPacks;
+  constexpr int kSteps = BM / kRowsPerStep;
+  static_assert(NT % kRowPacks == 0 && BM % kRowsPerStep == 0 && kSteps <= 32,
+                "output tile must split evenly over the threads");
+  const int pk = tid % kRowPacks, r0 = tid / kRowPacks;
+  const T* sp = stage_c + r0 * kLdc + pk * 8;
+  // Rows past the expert's last one are cut off by the buffer descriptor (the
+  // bytes of this tile end with the last valid row), so the loop carries no
+  // per-row condition.
+  const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(C + (int64_t)m0 * ldc + n0), (short)0, ((m_valid - 1) * ldc + n_valid) * 2,
+      kRsrcFlags);
+  const int c_off = (r0 * ldc + pk * 8) * 2;
+  if (n0 + pk * 8 < N) {  // N is a multiple of 8: a pack is all in or all out
+    // Every pack gets registers of its own: a store holds its data registers
+    // until memory has acknowledged it, so a register reused for a later pack
+    // would make that pack wait for a full store round trip.
+    i32x4_t v[kSteps];
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u)
+      v[u] = *reinterpret_cast<const i32x4_t*>(sp + u * kRowsPerStep * kLdc);
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u)
+      __builtin_amdgcn_raw_buffer_store_b128(v[u], c_rsrc, c_off + u * kRowsPerStep * ldc * 2, 0,
+                                             0);
   }
 }
 
