@@ -27,8 +27,8 @@
 // while one feeds the MFMAs; one barrier per slice.
 //
 // The rows of an expert are cut into BM-row tiles plus, for a remainder of at
-// most BM / 2 rows, 64-row tiles that cost a fraction of a BM tile, so a few
-// rows past a multiple of BM do not cost a whole tile.  Tiles are dealt to the
+// most BM / 2 rows, one 64- or 128-row tile that costs a fraction of a BM tile,
+// so a few rows past a multiple of BM do not cost a whole tile.  Tiles are dealt to the
 // workgroups in an XCD-aware patch order.
 //
 // Operand roles follow cuda/parallel_linear.cuh:69-87,124-147 of the
@@ -555,9 +555,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, Til
   }
 }
 
-// Remainder tiles (see the kernels below): 64 rows, K slices of 32 in 6 LDS
-// stages.  A slice of such a tile is a quarter of the MFMA work of a 256-row
-// one, so its copies need more slices of lead to cover the memory latency.
+// Remainder tiles (see the kernels below): 64 rows (the 4 waves side by side,
+// K slices of 32 in 6 LDS stages: a slice is a quarter of the MFMA work of a
+// 256-row one, so its copies need more slices of lead to cover the memory
+// latency) or 128 rows (2 x 2 waves, 4 stages).
 constexpr int kSmallRows = 64;
 constexpr int kSmallBK = 32;
 constexpr int kSmallStages = 6;
@@ -571,9 +572,10 @@ constexpr bool has_small_tiles() {
 }
 
 // How expert rows are cut into tiles: `full` tiles of BM rows from row 0 on
-// and, behind them, `small` tiles of kSmallRows rows.  A remainder of more than
-// BM / 2 rows takes one more BM tile; a shorter one is covered by small tiles,
-// which cost a fraction of a BM tile instead of a whole one.
+// and, for a remainder of at most BM / 2 rows, one remainder tile (`small` is
+// 0 or 1) of 64 rows, or of 128 rows when the remainder is longer than 64;
+// a remainder above BM / 2 rows takes one more BM tile.  Remainder tiles cost
+// about 0.45 (64 rows) and 0.6 (128 rows) of a 256-row tile.
 template <int BM, bool SMALL>
 __device__ __forceinline__ void cut_rows(int cnt, int& full, int& small) {
   if (!SMALL) {
@@ -583,9 +585,21 @@ __device__ __forceinline__ void cut_rows(int cnt, int& full, int& small) {
   }
   full = cnt / BM;
   const int rem = cnt - full * BM;
-  small = 0;
+  small = rem > 0 && rem <= BM / 2;
   if (rem > BM / 2) ++full;
-  else small = (rem + kSmallRows - 1) / kSmallRows;
+}
+
+// Runs the remainder tile at rows [where.m0, where.cnt) of its expert.
+template <typename T, int BM, int BN, int MODE>
+__device__ __forceinline__ void remainder_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
+                                               int n_tile) {
+  if constexpr (BM >= 4 * kSmallRows) {
+    if (where.cnt - where.m0 > kSmallRows) {
+      gemm_tile<T, 2 * kSmallRows, BN, kSmallBK, 2, 2, 4, MODE>(g, smem, where, n_tile);
+      return;
+    }
+  }
+  gemm_tile<T, kSmallRows, BN, kSmallBK, 1, 4, kSmallStages, MODE>(g, smem, where, n_tile);
 }
 
 // Position of a workgroup in the order in which tiles are handed out.
@@ -694,7 +708,7 @@ struct RowTiles {
       const int at = __builtin_amdgcn_readlane(first, owner);
       const int f = __builtin_amdgcn_readlane(mine_f, owner);
       t.e = owner;
-      t.m0 = small ? f * BM + (v - at) * kSmallRows : (v - at) * BM;
+      t.m0 = small ? f * BM : (v - at) * BM;
       t.row0 = __builtin_amdgcn_readlane(my_row0, owner);
       t.cnt = __builtin_amdgcn_readlane(my_cnt, owner);
       return t;
@@ -708,7 +722,7 @@ struct RowTiles {
         const int tx = small ? sm : f;
         if (v < at + tx) {
           s_out[0] = x;
-          s_out[1] = small ? f * BM + (v - at) * kSmallRows : (v - at) * BM;
+          s_out[1] = small ? f * BM : (v - at) * BM;
           s_out[2] = r0;
           s_out[3] = c;
           break;
@@ -762,7 +776,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   const TileRows where = rows.find(g.seg_off, v, small, s_owner);
   if constexpr (kSmall) {
     if (small) {
-      gemm_tile<T, kSmallRows, BN, kSmallBK, 1, NW, kSmallStages, MODE>(g, smem, where, n_tile);
+      remainder_tile<T, BM, BN, MODE>(g, smem, where, n_tile);
       return;
     }
   }
@@ -814,8 +828,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
   const TileRows where = rows.find(gd.seg_off, v, small, s_owner);
   if constexpr (kSmall) {
     if (small) {
-      gemm_tile<T, kSmallRows, BN, kSmallBK, 1, NW, kSmallStages, GEMM_DGRAD>(gd, smem, where,
-                                                                             n_tile);
+      remainder_tile<T, BM, BN, GEMM_DGRAD>(gd, smem, where, n_tile);
       return;
     }
   }
@@ -853,10 +866,8 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   } else {
     tiles_n = ceil_div(MODE == GEMM_FWD ? g.out_feat : g.in_feat, BN);
     // at most n_rows / BM whole tiles plus, per expert, one more BM tile or
-    // the small tiles of half a BM tile
-    constexpr int kPerExpert = has_small_tiles<BM, BN, MODE>() && BM / 2 > kSmallRows
-                                   ? BM / 2 / kSmallRows : 1;
-    tiles_m = (int)(g.n_rows / BM) + g.n_expert * kPerExpert;
+    // one remainder tile
+    tiles_m = (int)(g.n_rows / BM) + g.n_expert;
     blocks = (int64_t)tiles_n * tiles_m;
   }
   blocks = ceil_div(blocks, 8 * kXcdRun) * (8 * kXcdRun);  // whole runs for all 8 XCDs
@@ -944,16 +955,15 @@ static int launch_bwd_t(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
   }
   const int tiles_n_d = ceil_div(gd.in_feat, BN);
   const int tiles_n_w = ceil_div(gw.in_feat, BN), tiles_m_w = ceil_div(gw.out_feat, BM);
-  constexpr int kPerExpert = BM / 2 / kSmallRows;  // see launch_cfg
-  int64_t blocks = (int64_t)tiles_n_d * (gd.n_rows / BM + (int64_t)gd.n_expert * kPerExpert) +
+  int64_t blocks = (int64_t)tiles_n_d * (gd.n_rows / BM + (int64_t)gd.n_expert) +
                    (int64_t)tiles_n_w * tiles_m_w * gw.n_expert;
   blocks = ceil_div(blocks, 8 * kXcdRun) * (8 * kXcdRun);
   FMOE_REQUIRE(blocks < ((int64_t)1 << 31), FMOE_ERR_UNSUPPORTED,
                "grouped GEMM: too many tiles");
-  // a remainder tile walks out_feat values of K at about 0.34 us per 32, a dW
+  // a remainder tile walks out_feat values of K at about 0.4 us per 32, a dW
   // tile the rows of one expert at about 0.78 us per 32 (measured)
   const int small_first =
-      0.34 * gd.out_feat > 0.78 * (double)(gd.n_rows / gd.n_expert) ? 1 : 0;
+      0.4 * gd.out_feat > 0.78 * (double)(gd.n_rows / gd.n_expert) ? 1 : 0;
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NT), lds_bytes, s, gd, gw, tiles_n_d,
                      tiles_n_w, tiles_m_w, small_first);
   FMOE_LAUNCH_CHECK("gemm_bwd");
