@@ -108,8 +108,9 @@ class PresetGate(torch.nn.Module):
             if self.capacity is not None:
                 _l, _g, idx = limit_by_capacity(idx, self.num_expert, 1, self.capacity)
         else:
-            val, idx = torch.topk(self.logits, k=self.top_k, dim=-1, sorted=False)
-            score = F.softmax(val, dim=-1)
+            from fastmoe_amd.functions import topk_softmax
+
+            idx, score = topk_softmax(self.logits, self.top_k)
         return idx, score.to(self.dtype)
 
 
@@ -163,6 +164,8 @@ def kernel_work(cfg: dict, n_valid: int):
         "gather_combine_bwd": ("byte", T * d * s + 2.0 * n_valid * d * s + N * (4 + 2 * s)),
         "scatter_reduce": ("byte", n_valid * d * s + T * d * s + 4.0 * N),
         "expert_count": ("byte", 8.0 * N),
+        "topk_softmax_fwd": ("byte", 4.0 * T * E + 12.0 * N),
+        "topk_softmax_bwd": ("byte", 4.0 * T * E + 16.0 * N),
         "limit_by_capacity": ("byte", 20.0 * E),
         "prune_gate_by_capacity": ("byte", 24.0 * N),
     }

@@ -47,6 +47,10 @@ SIGNATURES = {
                                         c_void_p, c_void_p, c_void_p, c_int64,
                                         c_int64, c_int64, c_int64, c_int, c_void_p]),
     "fmoe_seg_off_from_host_counts": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
+    "fmoe_topk_softmax_fwd": (c_int, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p,
+                                      c_int, c_void_p]),
+    "fmoe_topk_softmax_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32,
+                                      c_int32, c_int, c_void_p]),
     "fmoe_set_gemm_path": (c_int, [c_int]),
 }
 
@@ -70,7 +74,7 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
         return _lib
     if not os.path.exists(LIB_PATH):
         if not build_if_missing:
-            raise ImportError(f"{LIB_PATH} is missing; run `python -m fastmoe_amd.build`")
+            raise ImportError(f"{LIB_PATH} is missing; run `python fastmoe_amd/build.py`")
         from . import build as _build
 
         _build.build(verbose=False)

@@ -1,6 +1,7 @@
 """Builds libfmoe_hip.so (HIP kernels + C ABI) for gfx950 with plain hipcc.
 
-Run as ``python -m fastmoe_amd.build``.  The library is torch-free; it is
+Run as ``python fastmoe_amd/build.py`` (as a script, so that a stale library
+from an earlier build is not loaded by the package import first).  The library is torch-free; it is
 written next to the package (fastmoe_amd/lib/) so a prebuilt copy travels with
 the source tree.  Building needs no GPU (hipcc cross-compiles).
 """
@@ -17,7 +18,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfmoe_hip.so")
 
-SOURCES = ["api.hip", "route.hip", "dispatch.hip", "gemm_simt.hip", "gemm_mfma.hip"]
+SOURCES = ["api.hip", "route.hip", "dispatch.hip", "gate.hip", "gemm_simt.hip", "gemm_mfma.hip"]
 HEADERS = ["common.h", "gemm.h", os.path.join("..", "..", "include", "fmoe_hip.h")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -49,7 +50,7 @@ def _compile(src: str, verbose: bool) -> str:
     return obj
 
 
-def build(verbose: bool = True, jobs: int = 5) -> str:
+def build(verbose: bool = True, jobs: int = 6) -> str:
     """Compiles every source and links the shared library; returns its path."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)

@@ -1,0 +1,229 @@
+// Top-k gate on gfx950: the k largest logits of every token and the softmax
+// over those k values in one pass, and the matching backward pass.
+//
+// Replaces the torch.topk + F.softmax pair of fmoe/gates/naive_gate.py:31-38
+// (and, in the backward, softmax-backward + zero-fill + scatter).  Results are
+// ordered by descending logit; equal logits go to the lower expert index.
+//
+// Eight lanes share a token (eight tokens per wave64): each lane keeps the k
+// best of every eighth logit in registers, then k rounds of a three-step
+// shuffle reduction pick the overall winners.  The arrays are a few hundred
+// KiB at most, so the kernels are launch-latency bound.
+#include "common.h"
+
+namespace fmoe {
+
+constexpr int kGateThreads = 256;
+constexpr int kGateLanes = 8;                       // lanes per token
+constexpr int kGateTokens = kGateThreads / kGateLanes;
+
+template <typename A>
+__device__ __forceinline__ bool better(A v, int e, A w, int f) {
+  return v > w || (v == w && e < f);
+}
+
+template <typename T, int KMAX>
+__global__ __launch_bounds__(kGateThreads) void topk_softmax_fwd_kernel(
+    const T* __restrict__ logits, int64_t n_tokens, int n_expert, int top_k,
+    int64_t* __restrict__ idx, T* __restrict__ score) {
+  using acc_t = typename Elem<T>::acc_t;
+  const int g = threadIdx.x % kGateLanes;
+  const int64_t t = (int64_t)blockIdx.x * kGateTokens + threadIdx.x / kGateLanes;
+  const bool live = t < n_tokens;
+  // local candidates, best first; empty slots hold (-inf, INT_MAX)
+  acc_t val[KMAX];
+  int id[KMAX];
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j) {
+    val[j] = -INFINITY;
+    id[j] = 0x7fffffff;
+  }
+  if (live) {
+    const T* row = logits + t * n_expert;
+    for (int e = g; e < n_expert; e += kGateLanes) {
+      acc_t v = Elem<T>::to_acc(row[e]);
+      int ve = e;
+      // insertion into the sorted list: the displaced entry moves down
+#pragma unroll
+      for (int j = 0; j < KMAX; ++j) {
+        if (better(v, ve, val[j], id[j])) {
+          const acc_t tv = val[j];
+          const int te = id[j];
+          val[j] = v;
+          id[j] = ve;
+          v = tv;
+          ve = te;
+        }
+      }
+    }
+  }
+  // k rounds: the best head of the eight lists wins and is popped
+  acc_t sel[KMAX];
+  int sel_id[KMAX];
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j) {
+    sel[j] = -INFINITY;
+    sel_id[j] = 0;
+    if (j < top_k) {
+      acc_t bv = val[0];
+      int be = id[0];
+#pragma unroll
+      for (int d = 1; d < kGateLanes; d <<= 1) {
+        const acc_t ov = __shfl_xor(bv, d, kWave);
+        const int oe = __shfl_xor(be, d, kWave);
+        if (better(ov, oe, bv, be)) {
+          bv = ov;
+          be = oe;
+        }
+      }
+      sel[j] = bv;
+      sel_id[j] = be;
+      if (id[0] == be) {  // this lane held the winner: pop it
+#pragma unroll
+        for (int q = 0; q + 1 < KMAX; ++q) {
+          val[q] = val[q + 1];
+          id[q] = id[q + 1];
+        }
+        val[KMAX - 1] = -INFINITY;
+        id[KMAX - 1] = 0x7fffffff;
+      }
+    }
+  }
+  if (!live || g != 0) return;
+  // softmax over the winners; sel[0] is the largest
+  acc_t p[KMAX];
+  acc_t sum = 0;
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j) {
+    p[j] = 0;
+    if (j < top_k) {
+      p[j] = exp(sel[j] - sel[0]);
+      sum += p[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j) {
+    if (j < top_k) {
+      idx[t * top_k + j] = sel_id[j];
+      score[t * top_k + j] = Elem<T>::from_acc(p[j] / sum);
+    }
+  }
+}
+
+// dlogits[t][idx[t][j]] = score_j * (dscore_j - sum_i dscore_i * score_i), zero elsewhere.
+template <typename T, int KMAX>
+__global__ __launch_bounds__(kGateThreads) void topk_softmax_bwd_kernel(
+    const T* __restrict__ dscore, const T* __restrict__ score,
+    const int64_t* __restrict__ idx, T* __restrict__ dlogits, int64_t n_tokens,
+    int n_expert, int top_k) {
+  using acc_t = typename Elem<T>::acc_t;
+  const int g = threadIdx.x % kGateLanes;
+  const int64_t t = (int64_t)blockIdx.x * kGateTokens + threadIdx.x / kGateLanes;
+  if (t >= n_tokens) return;
+  acc_t grad[KMAX];
+  int id[KMAX];
+  acc_t dot = 0;
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j) {
+    grad[j] = 0;
+    id[j] = -1;
+    if (j < top_k) {
+      const acc_t s = Elem<T>::to_acc(score[t * top_k + j]);
+      const acc_t d = Elem<T>::to_acc(dscore[t * top_k + j]);
+      dot += d * s;
+      grad[j] = d;
+      id[j] = (int)idx[t * top_k + j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j)
+    if (j < top_k) grad[j] = Elem<T>::to_acc(score[t * top_k + j]) * (grad[j] - dot);
+  T* row = dlogits + t * n_expert;
+  for (int e = g; e < n_expert; e += kGateLanes) {
+    acc_t v = 0;
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j)
+      if (id[j] == e) v = grad[j];
+    row[e] = Elem<T>::from_acc(v);
+  }
+}
+
+template <typename T, int KMAX>
+static int launch_fwd(const void* logits, int64_t n_tokens, int n_expert, int top_k,
+                      int64_t* idx, void* score, hipStream_t s) {
+  const int blocks = ceil_div(n_tokens, kGateTokens);
+  hipLaunchKernelGGL((topk_softmax_fwd_kernel<T, KMAX>), dim3(blocks), dim3(kGateThreads), 0, s,
+                     (const T*)logits, n_tokens, n_expert, top_k, idx, (T*)score);
+  FMOE_LAUNCH_CHECK("topk_softmax_fwd");
+  return FMOE_OK;
+}
+
+template <typename T, int KMAX>
+static int launch_bwd(const void* dscore, const void* score, const int64_t* idx, void* dlogits,
+                      int64_t n_tokens, int n_expert, int top_k, hipStream_t s) {
+  const int blocks = ceil_div(n_tokens, kGateTokens);
+  hipLaunchKernelGGL((topk_softmax_bwd_kernel<T, KMAX>), dim3(blocks), dim3(kGateThreads), 0, s,
+                     (const T*)dscore, (const T*)score, idx, (T*)dlogits, n_tokens, n_expert,
+                     top_k);
+  FMOE_LAUNCH_CHECK("topk_softmax_bwd");
+  return FMOE_OK;
+}
+
+static int check_gate(const char* who, int64_t n_tokens, int64_t n_expert, int64_t top_k,
+                      int dtype) {
+  FMOE_REQUIRE(dtype_size(dtype) != 0, FMOE_ERR_INVALID, "%s: unknown dtype %d", who, dtype);
+  FMOE_REQUIRE(n_tokens >= 0 && n_expert >= 1 && top_k >= 1, FMOE_ERR_INVALID,
+               "%s: bad sizes tokens=%lld experts=%lld top_k=%lld", who, (long long)n_tokens,
+               (long long)n_expert, (long long)top_k);
+  FMOE_REQUIRE(top_k <= n_expert, FMOE_ERR_INVALID, "%s: top_k %lld exceeds %lld experts", who,
+               (long long)top_k, (long long)n_expert);
+  FMOE_REQUIRE(top_k <= FMOE_MAX_GATE_TOP_K, FMOE_ERR_UNSUPPORTED,
+               "%s: top_k %lld exceeds FMOE_MAX_GATE_TOP_K (%d)", who, (long long)top_k,
+               FMOE_MAX_GATE_TOP_K);
+  FMOE_REQUIRE(n_expert < ((int64_t)1 << 31) &&
+                   n_tokens < ((int64_t)1 << 31) * kGateTokens,
+               FMOE_ERR_UNSUPPORTED, "%s: size exceeds the index range", who);
+  return FMOE_OK;
+}
+
+}  // namespace fmoe
+
+using namespace fmoe;
+
+#define FMOE_GATE_DISPATCH(FN, T, ...)                         \
+  (top_k <= 2 ? FN<T, 2>(__VA_ARGS__)                          \
+              : top_k <= 4 ? FN<T, 4>(__VA_ARGS__)             \
+                           : top_k <= 8 ? FN<T, 8>(__VA_ARGS__) : FN<T, 16>(__VA_ARGS__))
+
+extern "C" int fmoe_topk_softmax_fwd(const void* logits, int64_t n_tokens, int32_t n_expert,
+                                     int32_t top_k, int64_t* idx, void* score, int dtype,
+                                     void* stream) {
+  int rc = check_gate("topk_softmax_fwd", n_tokens, n_expert, top_k, dtype);
+  if (rc) return rc;
+  if (n_tokens == 0) return FMOE_OK;
+  FMOE_REQUIRE(logits && idx && score, FMOE_ERR_INVALID, "topk_softmax_fwd: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case FMOE_F32: return FMOE_GATE_DISPATCH(launch_fwd, float, logits, n_tokens, n_expert, top_k, idx, score, s);
+    case FMOE_F64: return FMOE_GATE_DISPATCH(launch_fwd, double, logits, n_tokens, n_expert, top_k, idx, score, s);
+    case FMOE_F16: return FMOE_GATE_DISPATCH(launch_fwd, __half, logits, n_tokens, n_expert, top_k, idx, score, s);
+    default: return FMOE_GATE_DISPATCH(launch_fwd, __hip_bfloat16, logits, n_tokens, n_expert, top_k, idx, score, s);
+  }
+}
+
+extern "C" int fmoe_topk_softmax_bwd(const void* dscore, const void* score, const int64_t* idx,
+                                     void* dlogits, int64_t n_tokens, int32_t n_expert,
+                                     int32_t top_k, int dtype, void* stream) {
+  int rc = check_gate("topk_softmax_bwd", n_tokens, n_expert, top_k, dtype);
+  if (rc) return rc;
+  if (n_tokens == 0) return FMOE_OK;
+  FMOE_REQUIRE(dscore && score && idx && dlogits, FMOE_ERR_INVALID,
+               "topk_softmax_bwd: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case FMOE_F32: return FMOE_GATE_DISPATCH(launch_bwd, float, dscore, score, idx, dlogits, n_tokens, n_expert, top_k, s);
+    case FMOE_F64: return FMOE_GATE_DISPATCH(launch_bwd, double, dscore, score, idx, dlogits, n_tokens, n_expert, top_k, s);
+    case FMOE_F16: return FMOE_GATE_DISPATCH(launch_bwd, __half, dscore, score, idx, dlogits, n_tokens, n_expert, top_k, s);
+    default: return FMOE_GATE_DISPATCH(launch_bwd, __hip_bfloat16, dscore, score, idx, dlogits, n_tokens, n_expert, top_k, s);
+  }
+}

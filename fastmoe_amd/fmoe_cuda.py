@@ -419,6 +419,45 @@ def scatter_reduce(dbuf: torch.Tensor, inv: torch.Tensor, n_tokens: int,
     return dx
 
 
+MAX_GATE_TOP_K = 16   # FMOE_MAX_GATE_TOP_K of the C ABI
+
+
+def topk_softmax_fwd(logits: torch.Tensor, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(idx int64 [T, k], score [T, k]) of logits [T, E]: the k largest logits of
+    every token by descending value (equal logits: lower index first) and the
+    softmax over them, as naive_gate.py:31-38 computes with torch.topk + softmax."""
+    _dev(logits, "logits")
+    _need(logits.dim() == 2, "logits must be [tokens, experts]")
+    t, e = logits.shape
+    idx = torch.empty((t, top_k), dtype=torch.int64, device=logits.device)
+    score = torch.empty((t, top_k), dtype=logits.dtype, device=logits.device)
+    with _launch(logits, "topk_softmax_fwd"):
+        _lib.check(
+            _L.fmoe_topk_softmax_fwd(logits.data_ptr(), t, e, top_k, idx.data_ptr(),
+                                     score.data_ptr(), _dt(logits, "logits"), _stream(logits)),
+            "topk_softmax_fwd")
+    return idx, score
+
+
+def topk_softmax_bwd(dscore: torch.Tensor, score: torch.Tensor, idx: torch.Tensor,
+                     n_expert: int) -> torch.Tensor:
+    """dlogits [T, E] of topk_softmax_fwd (zero outside the chosen experts)."""
+    _dev(dscore, "dscore")
+    _dev(score, "score", dscore.dtype)
+    _dev(idx, "idx", torch.int64)
+    t, k = score.shape
+    _need(tuple(dscore.shape) == (t, k) and tuple(idx.shape) == (t, k),
+          "dscore, score and idx must all be [tokens, top_k]")
+    dlogits = torch.empty((t, n_expert), dtype=score.dtype, device=score.device)
+    with _launch(score, "topk_softmax_bwd"):
+        _lib.check(
+            _L.fmoe_topk_softmax_bwd(dscore.data_ptr(), score.data_ptr(), idx.data_ptr(),
+                                     dlogits.data_ptr(), t, n_expert, k,
+                                     _dt(score, "score"), _stream(score)),
+            "topk_softmax_bwd")
+    return dlogits
+
+
 def set_gemm_path(path: int) -> None:
     """0 = matrix-core kernel where the shape allows (tile shape chosen by the
     library), 1 = scalar kernel only, 2..5 = matrix-core kernel with tile

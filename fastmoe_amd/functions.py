@@ -182,3 +182,35 @@ class FusedGatherCombine(Function):
         dbuf, dscore = fmoe_cuda.gather_combine_bwd(
             grad_y.contiguous(), buf, plan.inv, score, plan.n_tokens, plan.top_k)
         return dbuf, dscore.view_as(score), None
+
+
+class TopKSoftmax(Function):
+    r"""(idx, score) = top-k of the logits and the softmax over the k values,
+    the two torch calls of fmoe/gates/naive_gate.py:31-38 as one kernel each
+    way.  idx is ordered by descending logit and carries no gradient."""
+
+    @staticmethod
+    def forward(ctx, logits, top_k: int):
+        idx, score = fmoe_cuda.topk_softmax_fwd(logits.contiguous(), top_k)
+        ctx.n_expert = logits.shape[1]
+        ctx.save_for_backward(idx, score)
+        ctx.mark_non_differentiable(idx)
+        return idx, score
+
+    @staticmethod
+    def backward(ctx, _grad_idx, grad_score):
+        idx, score = ctx.saved_tensors
+        return fmoe_cuda.topk_softmax_bwd(grad_score.contiguous(), score, idx,
+                                          ctx.n_expert), None
+
+
+def topk_softmax(logits, top_k: int):
+    r"""Top-k gate decision of logits [..., E]: `(idx [T, k] int64, score [T, k])`.
+    On the GPU (and for k up to fmoe_cuda.MAX_GATE_TOP_K) one fused kernel; anywhere
+    else the torch.topk + softmax formulation of the reference."""
+    flat = logits.reshape(-1, logits.shape[-1])
+    if flat.is_cuda and top_k <= fmoe_cuda.MAX_GATE_TOP_K and flat.dtype in (
+            torch.float32, torch.float64, torch.float16, torch.bfloat16):
+        return TopKSoftmax.apply(flat, top_k)
+    val, idx = torch.topk(flat, k=top_k, dim=-1, largest=True, sorted=False)
+    return idx, torch.nn.functional.softmax(val, dim=-1)

@@ -1,8 +1,8 @@
 r"""Top-k of a linear layer (fmoe/gates/naive_gate.py)."""
 import torch
 import torch.nn as nn
-import torch.nn.functional as F
 
+from ..functions import topk_softmax
 from .base_gate import BaseGate
 
 
@@ -18,9 +18,7 @@ class NaiveGate(BaseGate):
 
     def forward(self, inp, return_all_scores=False):
         logits = self.gate(inp)
-        top_val, top_idx = torch.topk(logits, k=self.top_k, dim=-1, largest=True,
-                                      sorted=False)
-        score = F.softmax(top_val.view(-1, self.top_k), dim=-1)
+        top_idx, score = topk_softmax(logits, self.top_k)
         # a zero loss so training loops can always call get_loss()
         self.set_loss(torch.zeros(1, requires_grad=True).to(inp.device))
         if return_all_scores:

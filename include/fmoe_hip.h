@@ -51,6 +51,8 @@ typedef enum fmoe_dtype {
 
 /* Largest number of experts the routing kernels keep in LDS. */
 #define FMOE_MAX_EXPERTS 4096
+/* Largest top_k of the fused gate kernels. */
+#define FMOE_MAX_GATE_TOP_K 16
 
 /* Library identification and error text (thread-local, never NULL). */
 const char* fmoe_version(void);
@@ -224,6 +226,31 @@ int fmoe_grouped_linear_bwd(const void* dy, const void* x, const void* w,
 int fmoe_seg_off_from_host_counts(const int64_t* expert_count_host,
                                   int64_t n_expert, int32_t* seg_off,
                                   void* stream);
+
+/*
+ * Top-k gate in one pass: for every token the top_k largest of its n_expert
+ * logits (row-major logits[n_tokens][n_expert]) and the softmax over those
+ * top_k values:
+ *   idx[t][j]   = expert of the j-th largest logit (equal logits: lower index first)
+ *   score[t][j] = exp(v_j - v_0) / sum_i exp(v_i - v_0)      (dtype of the logits)
+ * Replaces torch.topk + F.softmax of fmoe/gates/naive_gate.py:31-38; torch.topk
+ * leaves the order of its results open, this call returns them by descending
+ * logit.  top_k <= min(n_expert, FMOE_MAX_GATE_TOP_K); NaN logits are never picked.
+ */
+int fmoe_topk_softmax_fwd(const void* logits, int64_t n_tokens, int32_t n_expert,
+                          int32_t top_k, int64_t* idx, void* score, int dtype,
+                          void* stream);
+
+/*
+ * Backward of fmoe_topk_softmax_fwd with respect to the logits:
+ *   dlogits[t][idx[t][j]] = score_j * (dscore_j - sum_i dscore_i * score_i)
+ * and zero for every other expert (all n_tokens * n_expert entries are written).
+ * Replaces the autograd chain of naive_gate.py:31-38 (softmax backward, zero
+ * fill, scatter of the top-k gradient).
+ */
+int fmoe_topk_softmax_bwd(const void* dscore, const void* score, const int64_t* idx,
+                          void* dlogits, int64_t n_tokens, int32_t n_expert,
+                          int32_t top_k, int dtype, void* stream);
 
 /*
  * Selects the grouped-GEMM kernel family for bf16/f16: 0 = automatic (MFMA

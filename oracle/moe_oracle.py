@@ -167,6 +167,33 @@ def linear_backward(dy, x, w, expert_count):
     return dx, dw, db
 
 
+# ------------------------------------------------------------------- gate
+def topk_softmax(logits: np.ndarray, top_k: int):
+    """fmoe/gates/naive_gate.py:31-38: the top_k largest logits of every row and
+    the softmax over those values, float64.  torch.topk leaves the order open;
+    here: descending logit, equal logits by ascending expert index."""
+    logits = np.asarray(logits, dtype=np.float64)
+    n_expert = logits.shape[1]
+    # stable sort of (-logit) keeps the lower index first among equals
+    order = np.argsort(-logits, axis=1, kind="stable")[:, :top_k]
+    val = np.take_along_axis(logits, order, axis=1)
+    p = np.exp(val - val[:, :1])
+    assert top_k <= n_expert
+    return order.astype(np.int64), p / p.sum(axis=1, keepdims=True)
+
+
+def topk_softmax_backward(dscore: np.ndarray, score: np.ndarray, idx: np.ndarray,
+                          n_expert: int) -> np.ndarray:
+    """Gradient of topk_softmax with respect to the logits: softmax backward on
+    the k chosen entries, zero elsewhere."""
+    dscore = np.asarray(dscore, dtype=np.float64)
+    score = np.asarray(score, dtype=np.float64)
+    g = score * (dscore - (dscore * score).sum(axis=1, keepdims=True))
+    out = np.zeros((score.shape[0], n_expert))
+    np.put_along_axis(out, np.asarray(idx), g, axis=1)
+    return out
+
+
 # ------------------------------------------------------- whole layer (torch)
 def brute_force_moe_mlp(inp, gate_idx, gate_score, w1, b1, w2, b2,
                         activation=F.gelu):

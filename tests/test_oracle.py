@@ -209,3 +209,28 @@ def test_brute_force_layer_matches_per_token_loop_and_k1_mlp():
     x.requires_grad_(True)
     O.brute_force_moe_mlp(x, idx, score, w1, b1, w2, b2).sum().backward()
     assert x.grad is not None and torch.isfinite(x.grad).all()
+
+
+def test_topk_softmax_against_torch_and_ties():
+    import torch
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(5)
+    logits = rng.standard_normal((37, 11))
+    idx, score = O.topk_softmax(logits, 3)
+    val, tidx = torch.topk(torch.from_numpy(logits), 3, dim=-1, largest=True, sorted=True)
+    assert (idx == tidx.numpy()).all()                    # no ties in random data
+    np.testing.assert_allclose(score, F.softmax(val, dim=-1).numpy(), rtol=1e-12)
+    # ties go to the lower index, -inf entries are never preferred to finite ones
+    tied = np.array([[1.0, 3.0, 3.0, -np.inf, 3.0], [0.0, 0.0, 0.0, 0.0, 0.0]])
+    idx, score = O.topk_softmax(tied, 2)
+    assert idx.tolist() == [[1, 2], [0, 1]]
+    np.testing.assert_allclose(score, [[0.5, 0.5], [0.5, 0.5]])
+    # backward against autograd of the torch formulation
+    lt = torch.from_numpy(logits).requires_grad_(True)
+    v, i = torch.topk(lt, 3, dim=-1)
+    sc = F.softmax(v, dim=-1)
+    g = torch.from_numpy(rng.standard_normal((37, 3)))
+    sc.backward(g)
+    got = O.topk_softmax_backward(g.numpy(), sc.detach().numpy(), i.numpy(), 11)
+    np.testing.assert_allclose(got, lt.grad.numpy(), rtol=1e-10, atol=1e-14)
