@@ -131,8 +131,8 @@ def test_errors_are_runtime_errors():
 
 @pytest.mark.parametrize("cfg", ["cfg2", "cfg5"])
 def test_full_size_gemm_properties(cfg):
-    """BASELINE-sized grouped GEMMs checked through properties that do not need
-    a CPU evaluation: agreement with fp32 matmul of sampled rows, exact zeros
+    """Full-size grouped GEMMs (the balanced and the fine-grained workload)
+    checked through properties that do not need a CPU evaluation: agreement with fp32 matmul of sampled rows, exact zeros
     for empty experts, and linearity in the input."""
     from fastmoe_amd import fmoe_cuda
 
