@@ -16,7 +16,7 @@
 //     [row][BK]; pack index XOR ((row ^ row/8) & 7); a lane reads its 8
 //     consecutive K values with one ds_read_b128.
 //   * K strided in memory (W in DGRAD, both operands in WGRAD): LDS is
-//     [k][rows] as it arrives; 32-byte segment index XOR (k & 3); fragments
+//     [k][rows] as it arrives; 32-byte segment index XOR 2 (k & 3); fragments
 //     come back through ds_read_b64_tr_b16, which transposes 16-bit elements
 //     across groups of 16 lanes.
 // Out-of-range packs (ragged M, N or K edges) are pointed beyond the buffer
@@ -75,6 +75,7 @@ struct DmaTile {
   static constexpr int kBlocks = kBytes / 1024;     // one wave instruction each
   static constexpr int kPerWave = kBlocks / NW;
   static_assert(kBlocks % NW == 0 && kPerWave >= 1, "tile must split evenly");
+  static_assert(KC || R >= 128, "the [k][rows] swizzle permutes 8 segments of 16 rows");
   static_assert(BK == 64 || BK == 32, "swizzles below assume 128- or 64-byte [row][BK] rows");
   static constexpr int kRowPacks = R / 8;           // packs per [k] row (KC == false)
   static constexpr int kKPacks = BK / 8;            // packs per [row] row (KC == true)
@@ -112,7 +113,7 @@ struct DmaTile {
         voff[i] = (uint32_t)(row * ld + pack_k(b, lane)) * 2u;
       } else {
         const int k = b * (64 / kRowPacks) + lane / kRowPacks;
-        const int rc = (lane % kRowPacks) ^ ((k & 3) << 1);
+        const int rc = (lane % kRowPacks) ^ ((k & 3) << 2);  // 32-byte segment ^ 2 (k & 3)
         voff[i] = rc * 8 < r_valid ? (uint32_t)(k * ld + rc * 8) * 2u : kOutOfRange;
       }
     }
@@ -181,7 +182,10 @@ struct DmaTile {
       // elements [k + i/4][m + 4*(i%4) .. +3] and receives [k .. k+3][m + i].
       const int k = kk * 16 + 8 * (lane >> 5) + ((lane & 15) >> 2);
       const int m = row32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-      const int seg = (m >> 4) ^ (k & 3), within = m & 15;   // 32-byte segments
+      // 32-byte segments; a 64-bit read is served 32 lanes at a time, i.e. 4 k-rows
+      // x 2 segments: XOR with 2 (k & 3) puts those 8 chunks into 8 different
+      // segments of a 256-byte bank row
+      const int seg = (m >> 4) ^ ((k & 3) << 1), within = m & 15;
       const uint16_t* p = lds + k * R + seg * 16 + within;
       const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
           (__attribute__((address_space(3))) s16x4_t*)(p));
