@@ -195,10 +195,13 @@ class TopKSoftmax(Function):
         ctx.n_expert = logits.shape[1]
         ctx.save_for_backward(idx, score)
         ctx.mark_non_differentiable(idx)
+        ctx.set_materialize_grads(False)   # no zero tensor for idx's "gradient"
         return idx, score
 
     @staticmethod
     def backward(ctx, _grad_idx, grad_score):
+        if grad_score is None:
+            return None, None
         idx, score = ctx.saved_tensors
         return fmoe_cuda.topk_softmax_bwd(grad_score.contiguous(), score, idx,
                                           ctx.n_expert), None
