@@ -914,10 +914,10 @@ template <typename T, int MODE>
 static int launch_mode(const GemmArgs& g, hipStream_t s) {
   switch (pick_tile<MODE>(g)) {
     case 1:
-      // Both FWD operands are [row][k] in memory: K slices of 64 move whole
-      // 128-byte lines and measured 7-8% faster there; the products with a
-      // [k][row] operand do as well or better with four stages of 32.
-      if (MODE == GEMM_FWD) return launch_cfg<T, 256, 256, 64, 2, 2, 2, MODE>(g, s);
+      // A [row][k] operand (both in FWD, dY in DGRAD) moves whole 128-byte
+      // lines with K slices of 64: measured 7-8% faster for FWD, 2% for DGRAD;
+      // WGRAD, with two [k][row] operands, is level with four stages of 32.
+      if (MODE != GEMM_WGRAD) return launch_cfg<T, 256, 256, 64, 2, 2, 2, MODE>(g, s);
       return launch_cfg<T, 256, 256, 32, 2, 2, 4, MODE>(g, s);
     case 2: return launch_cfg<T, 128, 256, 32, 2, 2, 4, MODE>(g, s);
     case 4: return launch_cfg<T, 256, 256, 64, 2, 2, 2, MODE>(g, s);
@@ -934,15 +934,10 @@ static int launch_t(int mode, const GemmArgs& g, hipStream_t s) {
   }
 }
 
-// dX and dW in one launch when both products would use the 256x256 tiles
-// anyway; otherwise one launch each.
-template <typename T>
-static int launch_bwd_t(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
-  if (pick_tile<GEMM_DGRAD>(gd) != 1 || pick_tile<GEMM_WGRAD>(gw) != 1) {
-    const int rc = launch_mode<T, GEMM_DGRAD>(gd, s);
-    return rc ? rc : launch_mode<T, GEMM_WGRAD>(gw, s);
-  }
-  constexpr int BM = 256, BN = 256, BK = 32, WM = 2, WN = 2, NS = 4, NT = WM * WN * 64;
+// dX and dW of one linear in one launch of 256x256 tiles, K slices of BK in NS stages.
+template <typename T, int BK, int NS>
+static int launch_bwd_fused(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
+  constexpr int BM = 256, BN = 256, WM = 2, WN = 2, NT = WM * WN * 64;
   constexpr size_t pipe_bytes = (size_t)NS * (BM + BN) * BK * 2;
   constexpr size_t out_bytes = (size_t)BM * (BN + 8) * 2;
   constexpr size_t small_bytes = (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2;
@@ -972,6 +967,23 @@ static int launch_bwd_t(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
                      tiles_n_w, tiles_m_w, small_first);
   FMOE_LAUNCH_CHECK("gemm_bwd");
   return FMOE_OK;
+}
+
+// dX and dW in one launch when both products would use the 256x256 tiles
+// anyway; otherwise one launch each.
+template <typename T>
+static int launch_bwd_t(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
+  const int pd = pick_tile<GEMM_DGRAD>(gd), pw = pick_tile<GEMM_WGRAD>(gw);
+  if (pd == 4 && pw == 4) return launch_bwd_fused<T, 64, 2>(gd, gw, s);  // forced
+  if (pd != 1 || pw != 1) {
+    const int rc = launch_mode<T, GEMM_DGRAD>(gd, s);
+    return rc ? rc : launch_mode<T, GEMM_WGRAD>(gw, s);
+  }
+  // K slices of 64 in two stages measured 2-3% faster than four stages of 32
+  // when dW's K (the rows of an expert) is long, 2% slower at ~500 rows
+  if (gd.tile != 1 && gd.n_rows / gd.n_expert >= 1024)
+    return launch_bwd_fused<T, 64, 2>(gd, gw, s);
+  return launch_bwd_fused<T, 32, 4>(gd, gw, s);
 }
 
 bool gemm_mfma_supported(int mode, const GemmArgs& g, int dtype) {
