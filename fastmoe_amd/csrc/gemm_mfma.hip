@@ -230,11 +230,11 @@ struct TileRows {
 };
 
 // One output tile: rows [m0, m0 + BM) of expert e's row range (WGRAD: of its
-// out_feat x in_feat gradient) by columns [n_tile * BN, + BN); `where` names
+// out_feat x in_feat gradient) by columns [n_origin, + BN); `where` names
 // the expert, m0 and the expert's rows.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
-                                          int n_tile) {
+                                          int n_origin) {
   constexpr int NW = WM * WN;
   constexpr int NT = NW * 64;
   constexpr bool A_KC = MODE != GEMM_WGRAD;
@@ -278,7 +278,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, Til
     C = (T*)g.c + (int64_t)e * out_f * in_f;                ldc = in_f;
   }
   const int m0 = __builtin_amdgcn_readfirstlane(where.m0);
-  const int n0 = __builtin_amdgcn_readfirstlane(n_tile) * BN;
+  const int n0 = __builtin_amdgcn_readfirstlane(n_origin);
   if (m0 >= M || n0 >= N) return;
   const int m_valid = min(BM, M - m0), n_valid = min(BN, N - n0);
 
@@ -593,17 +593,39 @@ __device__ __forceinline__ void cut_rows(int cnt, int& full, int& small) {
   if (rem > BM / 2) ++full;
 }
 
+// Runs a BM x BN tile, or the half-width / half-height tile that covers it when
+// at most half of its columns (any product) or of its rows (WGRAD: the rows of
+// dW are out_feat) exist: a feature size of, say, 1408 = 5.5 x 256 then pays
+// for 5.6 tiles instead of 6.
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
+__device__ __forceinline__ void edge_aware_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
+                                                int n_tile) {
+  const int n0 = n_tile * BN;
+  if constexpr (BM == 256 && BN == 256 && WM == 2 && WN == 2) {
+    const int n_total = MODE == GEMM_FWD ? g.out_feat : g.in_feat;
+    if (n_total - n0 <= BN / 2) {
+      gemm_tile<T, BM, BN / 2, BK, WM, WN, NS, MODE>(g, smem, where, n0);
+      return;
+    }
+    if (MODE == GEMM_WGRAD && g.out_feat - where.m0 <= BM / 2) {
+      gemm_tile<T, BM / 2, BN, 32, WM, WN, 4, MODE>(g, smem, where, n0);
+      return;
+    }
+  }
+  gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, where, n0);
+}
+
 // Runs the remainder tile at rows [where.m0, where.cnt) of its expert.
 template <typename T, int BM, int BN, int MODE>
 __device__ __forceinline__ void remainder_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
                                                int n_tile) {
   if constexpr (BM >= 4 * kSmallRows) {
     if (where.cnt - where.m0 > kSmallRows) {
-      gemm_tile<T, 2 * kSmallRows, BN, kSmallBK, 2, 2, 4, MODE>(g, smem, where, n_tile);
+      gemm_tile<T, 2 * kSmallRows, BN, kSmallBK, 2, 2, 4, MODE>(g, smem, where, n_tile * BN);
       return;
     }
   }
-  gemm_tile<T, kSmallRows, BN, kSmallBK, 1, 4, kSmallStages, MODE>(g, smem, where, n_tile);
+  gemm_tile<T, kSmallRows, BN, kSmallBK, 1, 4, kSmallStages, MODE>(g, smem, where, n_tile * BN);
 }
 
 // Position of a workgroup in the order in which tiles are handed out.
@@ -763,8 +785,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
     tile_order(t % (tiles_n * tiles_m), tiles_m, tiles_n, m_tile, n_tile);
     const int e = t / (tiles_n * tiles_m);
     const int row0 = g.seg_off[e];
-    gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, {e, m_tile * BM, row0, g.seg_off[e + 1] - row0},
-                                                n_tile);
+    edge_aware_tile<T, BM, BN, BK, WM, WN, NS, MODE>(
+        g, smem, {e, m_tile * BM, row0, g.seg_off[e + 1] - row0}, n_tile);
     return;
   }
   RowTiles<BM, kSmall, NW> rows;
@@ -784,7 +806,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
       return;
     }
   }
-  gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, where, n_tile);
+  edge_aware_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, where, n_tile);
 }
 
 // Both gradient products of one grouped linear in one launch: the BM-row
@@ -821,7 +843,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
     tile_order(tw % per_expert_w, tiles_m_w, tiles_n_w, m_tile, n_tile);
     const int e = tw / per_expert_w;
     const int row0 = gw.seg_off[e];
-    gemm_tile<T, BM, BN, BK, WM, WN, NS, GEMM_WGRAD>(
+    edge_aware_tile<T, BM, BN, BK, WM, WN, NS, GEMM_WGRAD>(
         gw, smem, {e, m_tile * BM, row0, gw.seg_off[e + 1] - row0}, n_tile);
     return;
   }
@@ -836,7 +858,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
       return;
     }
   }
-  gemm_tile<T, BM, BN, BK, WM, WN, NS, GEMM_DGRAD>(gd, smem, where, n_tile);
+  edge_aware_tile<T, BM, BN, BK, WM, WN, NS, GEMM_DGRAD>(gd, smem, where, n_tile);
 }
 
 // ------------------------------------------------------------------ host side

@@ -82,6 +82,7 @@ FORCED = [
     ([300, 0, 257, 64, 1, 200, 513], 136, 264),
     ([1024 + 17, 1024 - 9, 0, 130], 72, 520),
     ([255, 129, 128, 65, 63], 264, 256),
+    ([520, 260, 0, 256], 352, 384),         # last column tile exactly / under half a tile
 ]
 
 
