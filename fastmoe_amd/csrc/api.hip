@@ -116,6 +116,8 @@ static int check_linear(const char* who, int64_t n_rows, int64_t in_feat,
 static int run_gemm(int mode, const GemmArgs& g, int dtype, hipStream_t s) {
   if (g_gemm_path == 0 && gemm_mfma_supported(mode, g, dtype))
     return launch_gemm_mfma(mode, g, dtype, s);
+  if (g_gemm_path == 0 && gemm_mfma_wide_supported(mode, g, dtype))
+    return launch_gemm_mfma_wide(mode, g, dtype, s);
   return launch_gemm_simt(mode, g, dtype, s);
 }
 

@@ -1,0 +1,324 @@
+// f32 / f64 grouped GEMM on the matrix cores (v_mfma_f32_32x32x2_f32,
+// v_mfma_f64_16x16x4_f64): the full-precision half of the reference's dtype
+// dispatch (cuda/parallel_linear.cu:33,76 -> cublasSgemm / cublasDgemm,
+// cuda/utils/cublas_wrapper.h:51-90).
+//
+// These MFMAs run at 1/16 (f32) and 1/32 (f64) of the bf16 rate, so one K slice
+// of a 128x128 tile keeps the matrix cores busy for microseconds and a plain
+// design is enough: global -> registers -> LDS with two LDS stages, one barrier
+// per slice, two blocks per CU so that one block's barrier and LDS writes hide
+// behind the other's MFMAs.  Operand roles and the ragged rows are those of the
+// bf16 kernel (gemm.h); the row tiles of an expert are found as in the scalar
+// kernel (virtual_row_tiles).
+//
+// LDS holds both operands K-major, [k][row], so the MFMA operand of a lane
+// (one value: row = lane % block, k = lane / block) is a conflict-free 4- or
+// 8-byte read.  Operands that are K-contiguous in memory (X and W in FWD, dY in
+// DGRAD) are transposed on the way in (4-element packs read along K, written
+// as 4 single values); the others are copied pack by pack.
+#include "gemm.h"
+
+namespace fmoe {
+namespace {
+
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef double f64x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kWideTile = 128;     // output tile is kWideTile x kWideTile
+constexpr int kWideThreads = 256;  // 2 x 2 waves of 64 x 64
+
+template <typename F> struct WideMma;
+template <> struct WideMma<float> {
+  static constexpr int kBlk = 32;   // rows / columns of one MFMA block
+  static constexpr int kStep = 2;   // values of K per MFMA
+  static constexpr int kAcc = 16;   // accumulators per lane and block
+  static constexpr int kBK = 16;    // values of K per LDS slice
+  static constexpr int kPad = 4;    // row padding of the LDS image, in elements
+  static constexpr int kWaves = 4;      // waves per SIMD the registers are budgeted for
+  static constexpr bool kSwap = true;   // feed (B, A): a lane then owns runs of 4 columns
+  using acc_t = f32x16_t;
+  typedef float vec_t __attribute__((ext_vector_type(4)));             // 16-byte pack
+  static __device__ __forceinline__ acc_t run(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct WideMma<double> {
+  static constexpr int kBlk = 16;
+  static constexpr int kStep = 4;
+  static constexpr int kAcc = 4;
+  static constexpr int kBK = 16;
+  static constexpr int kPad = 2;
+  static constexpr int kWaves = 2;
+  static constexpr bool kSwap = false;  // a lane owns one column, 16 lanes a row segment
+  using acc_t = f64x4_t;
+  typedef double vec_t __attribute__((ext_vector_type(4), aligned(16)));  // two 16-byte packs
+  static __device__ __forceinline__ acc_t run(double a, double b, acc_t c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename F>
+constexpr size_t wide_lds_bytes() {
+  return (size_t)2 * 2 * WideMma<F>::kBK * (kWideTile + WideMma<F>::kPad) * sizeof(F);
+}
+
+template <typename F, int MODE>
+__global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_kernel(GemmArgs g) {
+  using Mma = WideMma<F>;
+  constexpr int BK = Mma::kBK, BLK = Mma::kBlk, LD = kWideTile + Mma::kPad;
+  constexpr int kOperand = BK * LD;           // elements of one operand slice
+  constexpr int kVecs = BK * kWideTile / 4 / kWideThreads;   // packs per thread and operand
+  constexpr int TB = 64 / BLK;                // MFMA blocks per wave and direction
+  constexpr bool A_KC = MODE != GEMM_WGRAD;   // operand is K-contiguous in memory
+  constexpr bool B_KC = MODE == GEMM_FWD;
+  using Vec4 = typename Mma::vec_t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  F* smem = reinterpret_cast<F*>(smem_raw);   // [stage][A | B][k][row]
+  __shared__ int s_expert;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+  const int in_f = g.in_feat, out_f = g.out_feat;
+  int e, m_tile;
+  if (MODE == GEMM_WGRAD) {
+    e = blockIdx.z;
+    m_tile = blockIdx.y;
+  } else {
+    // the expert that owns virtual row tile blockIdx.y
+    const int v = blockIdx.y;
+    if (tid == 0) {
+      int lo = 0, hi = g.n_expert - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (g.seg_off[mid] / kWideTile + mid <= v) lo = mid; else hi = mid - 1;
+      }
+      s_expert = lo;
+    }
+    __syncthreads();
+    e = s_expert;
+    m_tile = v - (g.seg_off[e] / kWideTile + e);
+  }
+  const int64_t row0 = g.seg_off[e];
+  const int cnt = g.seg_off[e + 1] - g.seg_off[e];
+
+  int M, N, K, lda, ldb, ldc;
+  const F *A, *B;
+  F* C;
+  if (MODE == GEMM_FWD) {
+    M = cnt; N = out_f; K = in_f;
+    A = (const F*)g.a + row0 * in_f;                 lda = in_f;
+    B = (const F*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
+    C = (F*)g.c + row0 * out_f;                      ldc = out_f;
+  } else if (MODE == GEMM_DGRAD) {
+    M = cnt; N = in_f; K = out_f;
+    A = (const F*)g.a + row0 * out_f;                lda = out_f;
+    B = (const F*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
+    C = (F*)g.c + row0 * in_f;                       ldc = in_f;
+  } else {
+    M = out_f; N = in_f; K = cnt;
+    A = (const F*)g.a + row0 * out_f;                lda = out_f;
+    B = (const F*)g.b + row0 * in_f;                 ldb = in_f;
+    C = (F*)g.c + (int64_t)e * out_f * in_f;         ldc = in_f;
+  }
+  const int m0 = m_tile * kWideTile, n0 = blockIdx.x * kWideTile;
+  if (m0 >= M || n0 >= N) return;  // the same for the whole block
+  const int m_valid = min(kWideTile, M - m0), n_valid = min(kWideTile, N - n0);
+  const F* a_base = A_KC ? A + (int64_t)m0 * lda : A + m0;
+  const F* b_base = B_KC ? B + (int64_t)n0 * ldb : B + n0;
+
+  // Slice [k0, k0 + BK) of one operand into registers; rows past `valid` and
+  // values of K past the end arrive as zeros.  K-contiguous operands need K to
+  // be a multiple of 4, the others `valid` (a feature size) to be one.
+  auto fetch = [&](Vec4* r, const F* base, int ld, auto kc_tag, int valid, int k0) {
+    constexpr bool kc = decltype(kc_tag)::value;
+#pragma unroll
+    for (int u = 0; u < kVecs; ++u) {
+      const int idx = tid + u * kWideThreads;
+      bool ok;
+      const F* p;
+      if (kc) {
+        const int row = idx / (BK / 4), kq = idx % (BK / 4);
+        ok = row < valid && k0 + 4 * kq < K;
+        p = base + (int64_t)row * ld + k0 + 4 * kq;
+      } else {
+        const int k = idx / (kWideTile / 4), q = idx % (kWideTile / 4);
+        ok = k0 + k < K && 4 * q < valid;
+        p = base + (int64_t)(k0 + k) * ld + 4 * q;
+      }
+      r[u] = 0;
+      if (ok) r[u] = *reinterpret_cast<const Vec4*>(p);
+    }
+  };
+  auto stash = [&](const Vec4* r, F* dst, auto kc_tag) {
+    constexpr bool kc = decltype(kc_tag)::value;
+#pragma unroll
+    for (int u = 0; u < kVecs; ++u) {
+      const int idx = tid + u * kWideThreads;
+      if (kc) {
+        const int row = idx / (BK / 4), kq = idx % (BK / 4);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) dst[(4 * kq + c) * LD + row] = r[u][c];
+      } else {
+        const int k = idx / (kWideTile / 4), q = idx % (kWideTile / 4);
+        *reinterpret_cast<Vec4*>(dst + k * LD + 4 * q) = r[u];
+      }
+    }
+  };
+  using a_kc = std::integral_constant<bool, A_KC>;
+  using b_kc = std::integral_constant<bool, B_KC>;
+
+  // f32: acc[i][j] holds the TRANSPOSE of block (i, j) of C (the MFMA is fed
+  // (B value, A value)): a lane owns row lane % 32 and runs of 4 consecutive
+  // columns, which leave as one 16-byte store each.  f64: block (i, j) itself.
+  typename Mma::acc_t acc[TB][TB];
+#pragma unroll
+  for (int i = 0; i < TB; ++i)
+#pragma unroll
+    for (int j = 0; j < TB; ++j)
+#pragma unroll
+      for (int r = 0; r < Mma::kAcc; ++r) acc[i][j][r] = 0;
+
+  Vec4 ra[kVecs], rb[kVecs];
+  const int k_tiles = (K + BK - 1) / BK;
+  if (k_tiles > 0) {
+    fetch(ra, a_base, lda, a_kc{}, m_valid, 0);
+    fetch(rb, b_base, ldb, b_kc{}, n_valid, 0);
+    stash(ra, smem, a_kc{});
+    stash(rb, smem + kOperand, b_kc{});
+  }
+  __syncthreads();
+  const int lr = lane % BLK, lk = lane / BLK;
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const F* as = smem + (kt & 1) * 2 * kOperand;
+    const F* bs = as + kOperand;
+    const bool more = kt + 1 < k_tiles;
+    if (more) {  // in flight while this slice is multiplied
+      fetch(ra, a_base, lda, a_kc{}, m_valid, (kt + 1) * BK);
+      fetch(rb, b_base, ldb, b_kc{}, n_valid, (kt + 1) * BK);
+    }
+#pragma unroll
+    for (int kk = 0; kk < BK / Mma::kStep; ++kk) {
+      F a[TB], b[TB];
+#pragma unroll
+      for (int i = 0; i < TB; ++i)
+        a[i] = as[(kk * Mma::kStep + lk) * LD + wave_m * 64 + i * BLK + lr];
+#pragma unroll
+      for (int j = 0; j < TB; ++j)
+        b[j] = bs[(kk * Mma::kStep + lk) * LD + wave_n * 64 + j * BLK + lr];
+#pragma unroll
+      for (int i = 0; i < TB; ++i)
+#pragma unroll
+        for (int j = 0; j < TB; ++j)
+          acc[i][j] = Mma::kSwap ? Mma::run(b[j], a[i], acc[i][j]) : Mma::run(a[i], b[j], acc[i][j]);
+    }
+    if (more) {
+      // the other stage was last read in iteration kt - 1, which every wave
+      // left through the barrier below
+      F* next = smem + ((kt + 1) & 1) * 2 * kOperand;
+      stash(ra, next, a_kc{});
+      stash(rb, next + kOperand, b_kc{});
+    }
+    __syncthreads();
+  }
+
+  const F* bias = (MODE == GEMM_FWD && g.bias) ? (const F*)g.bias + (int64_t)e * out_f : nullptr;
+  if constexpr (Mma::kSwap) {
+    // 32x32 block, operands swapped: accumulator r of a lane is row lane % 32,
+    // column 8 * (r / 4) + 4 * (lane / 32) + r % 4
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      const int m = m0 + wave_m * 64 + i * BLK + lr;
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+#pragma unroll
+        for (int q = 0; q < Mma::kAcc / 4; ++q) {
+          const int n = n0 + wave_n * 64 + j * BLK + 8 * q + 4 * lk;
+          if (m < M && n < N) {  // N is a multiple of 4
+            Vec4 o;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) o[c] = acc[i][j][4 * q + c] + (bias ? bias[n + c] : (F)0);
+            *reinterpret_cast<Vec4*>(C + (int64_t)m * ldc + n) = o;
+          }
+        }
+      }
+    }
+  } else {
+    // 16x16 block: accumulator r of a lane is row 4 * r + lane / 16, column
+    // lane % 16; 16 lanes store 128 contiguous bytes of a row
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+      const int n = n0 + wave_n * 64 + j * BLK + lr;
+      const F bv = bias && n < N ? bias[n] : (F)0;
+#pragma unroll
+      for (int i = 0; i < TB; ++i) {
+#pragma unroll
+        for (int r = 0; r < Mma::kAcc; ++r) {
+          const int m = m0 + wave_m * 64 + i * BLK + 4 * r + lk;
+          if (m < M && n < N) C[(int64_t)m * ldc + n] = acc[i][j][r] + bv;
+        }
+      }
+    }
+  }
+}
+
+template <typename F, int MODE>
+int launch_wide_mode(const GemmArgs& g, hipStream_t s) {
+  constexpr size_t lds = wide_lds_bytes<F>();
+  static_assert(2 * (lds + 64) <= 160 * 1024, "two blocks per gfx950 CU");
+  auto kern = gemm_wide_kernel<F, MODE>;
+  static bool configured = false;  // attribute is per function, set once
+  if (!configured) {
+    FMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    configured = true;
+  }
+  dim3 grid;
+  if (MODE == GEMM_WGRAD) {
+    grid = dim3(ceil_div(g.in_feat, kWideTile), ceil_div(g.out_feat, kWideTile), g.n_expert);
+    FMOE_REQUIRE(grid.y <= 65535 && grid.z <= 65535, FMOE_ERR_UNSUPPORTED,
+                 "grouped GEMM: grid too large");
+  } else {
+    const int vt = virtual_row_tiles(g.n_rows, g.n_expert, kWideTile);
+    grid = dim3(ceil_div(MODE == GEMM_FWD ? g.out_feat : g.in_feat, kWideTile), vt, 1);
+    FMOE_REQUIRE(grid.y <= 65535, FMOE_ERR_UNSUPPORTED,
+                 "grouped GEMM: too many row tiles (%d)", vt);
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(kWideThreads), lds, s, g);
+  FMOE_LAUNCH_CHECK("gemm_wide");
+  return FMOE_OK;
+}
+
+template <typename F>
+int launch_wide_t(int mode, const GemmArgs& g, hipStream_t s) {
+  switch (mode) {
+    case GEMM_FWD: return launch_wide_mode<F, GEMM_FWD>(g, s);
+    case GEMM_DGRAD: return launch_wide_mode<F, GEMM_DGRAD>(g, s);
+    default: return launch_wide_mode<F, GEMM_WGRAD>(g, s);
+  }
+}
+
+}  // namespace
+
+// The 128x128 tiles pay off once they fill the chip; below that the 64x64
+// tiles of the scalar kernel spread a small problem over more CUs.  A forced
+// tile configuration (tests, tuning) takes the matrix cores at any size.
+bool gemm_mfma_wide_supported(int mode, const GemmArgs& g, int dtype) {
+  if (dtype != FMOE_F32 && dtype != FMOE_F64) return false;
+  if (g.in_feat % 4 != 0 || g.out_feat % 4 != 0) return false;
+  if (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.c) % 16 != 0) return false;
+  if (g.tile != 0) return true;
+  const int64_t tiles = mode == GEMM_WGRAD
+      ? (int64_t)g.n_expert * ceil_div(g.out_feat, kWideTile) * ceil_div(g.in_feat, kWideTile)
+      : (g.n_rows / kWideTile) *
+            ceil_div(mode == GEMM_FWD ? g.out_feat : g.in_feat, kWideTile);
+  return tiles >= 256;
+}
+
+int launch_gemm_mfma_wide(int mode, const GemmArgs& g, int dtype, hipStream_t s) {
+  if (!gemm_mfma_wide_supported(mode, g, dtype))
+    return set_error(FMOE_ERR_UNSUPPORTED, "grouped GEMM: shape not MFMA-aligned");
+  if (dtype == FMOE_F32) return launch_wide_t<float>(mode, g, s);
+  return launch_wide_t<double>(mode, g, s);
+}
+
+}  // namespace fmoe
