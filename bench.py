@@ -166,6 +166,8 @@ def kernel_work(cfg: dict, n_valid: int):
         "expert_count": ("byte", 8.0 * N),
         "topk_softmax_fwd": ("byte", 4.0 * T * E + 12.0 * N),
         "topk_softmax_bwd": ("byte", 4.0 * T * E + 16.0 * N),
+        "gelu_fwd": ("byte", 2.0 * n_valid * h * s),
+        "gelu_bwd": ("byte", 3.0 * n_valid * h * s),
         "limit_by_capacity": ("byte", 20.0 * E),
         "prune_gate_by_capacity": ("byte", 24.0 * N),
     }

@@ -18,7 +18,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfmoe_hip.so")
 
-SOURCES = ["api.hip", "route.hip", "dispatch.hip", "gate.hip", "gemm_simt.hip", "gemm_mfma.hip",
+SOURCES = ["api.hip", "route.hip", "dispatch.hip", "gate.hip", "act.hip", "gemm_simt.hip", "gemm_mfma.hip",
            "gemm_mfma_wide.hip"]
 HEADERS = ["common.h", "gemm.h", os.path.join("..", "..", "include", "fmoe_hip.h")]
 

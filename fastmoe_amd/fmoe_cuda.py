@@ -458,6 +458,31 @@ def topk_softmax_bwd(dscore: torch.Tensor, score: torch.Tensor, idx: torch.Tenso
     return dlogits
 
 
+def gelu_fwd(x: torch.Tensor) -> torch.Tensor:
+    """gelu(x) = 0.5 x (1 + erf(x / sqrt 2)), the torch.nn.GELU() between the two
+    expert layers (fmoe/transformer.py:28-30)."""
+    _dev(x, "x")
+    _need(x.is_contiguous(), "x must be contiguous")
+    y = torch.empty_like(x)
+    with _launch(x, "gelu_fwd"):
+        _lib.check(_L.fmoe_gelu_fwd(x.data_ptr(), y.data_ptr(), x.numel(), _dt(x, "x"),
+                                    _stream(x)), "gelu_fwd")
+    return y
+
+
+def gelu_bwd(dy: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """dy * gelu'(x)."""
+    _dev(x, "x")
+    _dev(dy, "dy", x.dtype)
+    _need(x.is_contiguous() and dy.is_contiguous() and dy.numel() == x.numel(),
+          "dy and x must be contiguous and of one size")
+    dx = torch.empty_like(x)
+    with _launch(x, "gelu_bwd"):
+        _lib.check(_L.fmoe_gelu_bwd(dy.data_ptr(), x.data_ptr(), dx.data_ptr(), x.numel(),
+                                    _dt(x, "x"), _stream(x)), "gelu_bwd")
+    return dx
+
+
 def set_gemm_path(path: int) -> None:
     """0 = matrix-core kernel where the shape allows (tile shape chosen by the
     library), 1 = scalar kernel only, 2..5 = matrix-core kernel with bf16/f16

@@ -207,6 +207,33 @@ class TopKSoftmax(Function):
                                           ctx.n_expert), None
 
 
+class Gelu(Function):
+    r"""The exact (erf) GELU between the two expert layers, the
+    `self.activation(x)` of fmoe/transformer.py:28-30 for torch.nn.GELU(), as
+    one kernel each way."""
+
+    @staticmethod
+    def forward(ctx, x):
+        x = x.contiguous()
+        ctx.save_for_backward(x)
+        return fmoe_cuda.gelu_fwd(x)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        (x,) = ctx.saved_tensors
+        return fmoe_cuda.gelu_bwd(grad_y.contiguous(), x)
+
+
+def apply_activation(activation, x):
+    r"""`activation(x)`; an exact torch.nn.GELU on a GPU tensor runs as the
+    library's kernel, anything else as the module itself."""
+    if (type(activation) is torch.nn.GELU and getattr(activation, "approximate", "none") == "none"
+            and x.is_cuda and x.dtype in (torch.float32, torch.float64, torch.float16,
+                                          torch.bfloat16)):
+        return Gelu.apply(x)
+    return activation(x)
+
+
 def topk_softmax(logits, top_k: int):
     r"""Top-k gate decision of logits [..., E]: `(idx [T, k] int64, score [T, k])`.
     On the GPU (and for k up to fmoe_cuda.MAX_GATE_TOP_K) one fused kernel; anywhere

@@ -4,6 +4,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from .functions import apply_activation
 from .layers import FMoE
 from .linear import FMoELinear
 
@@ -23,7 +24,7 @@ class _Expert(nn.Module):
 
     def forward(self, inp, fwd_expert_count):
         x = self.htoh4(inp, fwd_expert_count)
-        x = self.activation(x)
+        x = apply_activation(self.activation, x)
         return self.h4toh(x, fwd_expert_count)
 
 

@@ -255,6 +255,21 @@ int fmoe_topk_softmax_bwd(const void* dscore, const void* score, const int64_t* 
                           int32_t top_k, int dtype, void* stream);
 
 /*
+ * y[i] = gelu(x[i]) = 0.5 x (1 + erf(x / sqrt 2)) over n elements, and
+ * dx[i] = dy[i] * gelu'(x[i]): the activation between the two expert layers,
+ * fmoe/transformer.py:28-30 with the default torch.nn.GELU() of
+ * transformer.py:45 (the reference calls the torch module; these kernels take
+ * its place on the GPU).  bf16/f16 read gelu(x) (computed in double precision,
+ * rounded once) and gelu'(-|x|) (f32) from tables held in LDS; f32/f64 evaluate
+ * erf.  Inputs and outputs must not overlap.  The first 16-bit call on a
+ * GPU builds that GPU's tables on `stream`; first calls on one GPU must not come
+ * from two streams at once.
+ */
+int fmoe_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream);
+int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, int dtype,
+                  void* stream);
+
+/*
  * Selects the grouped-GEMM kernel family: 0 = automatic (MFMA where the shape
  * allows, tile shape from the library's cost model), 1 = force the scalar
  * kernel, 2..5 = MFMA with bf16/f16 tile configuration 1..4 forced (256x256,

@@ -20,6 +20,7 @@ from ctypes import c_int64, c_void_p
 import numpy as np
 import torch
 import torch.nn.functional as F
+from scipy.special import erfc as _erfc
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libfmoe_oracle.so")
@@ -192,6 +193,22 @@ def topk_softmax_backward(dscore: np.ndarray, score: np.ndarray, idx: np.ndarray
     out = np.zeros((score.shape[0], n_expert))
     np.put_along_axis(out, np.asarray(idx), g, axis=1)
     return out
+
+
+# ------------------------------------------------------------- activation
+def gelu(x: np.ndarray) -> np.ndarray:
+    """The torch.nn.GELU() that fmoe/transformer.py:28-30 applies between the two
+    expert layers (default of transformer.py:45): x Phi(x), float64.  Phi through
+    erfc, which keeps the relative accuracy of the negative tail."""
+    x = np.asarray(x, dtype=np.float64)
+    return 0.5 * x * _erfc(-x / np.sqrt(2.0))
+
+
+def gelu_backward(dy: np.ndarray, x: np.ndarray) -> np.ndarray:
+    """dy * (Phi(x) + x phi(x)), float64."""
+    x = np.asarray(x, dtype=np.float64)
+    grad = 0.5 * _erfc(-x / np.sqrt(2.0)) + x * np.exp(-0.5 * x * x) / np.sqrt(2.0 * np.pi)
+    return np.asarray(dy, dtype=np.float64) * grad
 
 
 # ------------------------------------------------------- whole layer (torch)

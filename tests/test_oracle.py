@@ -234,3 +234,30 @@ def test_topk_softmax_against_torch_and_ties():
     sc.backward(g)
     got = O.topk_softmax_backward(g.numpy(), sc.detach().numpy(), i.numpy(), 11)
     np.testing.assert_allclose(got, lt.grad.numpy(), rtol=1e-10, atol=1e-14)
+
+
+def test_gelu_against_torch_and_identities():
+    import torch
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(11)
+    x = np.concatenate([rng.standard_normal(500) * 3, [0.0, -0.0, 1e-30, -40.0, 40.0, -8.5]])
+    want = F.gelu(torch.from_numpy(x)).numpy()                 # library routine, float64
+    # (torch evaluates 1 + erf, which cancels in the negative tail: absolute there)
+    np.testing.assert_allclose(O.gelu(x), want, rtol=1e-12, atol=2e-15)
+    # x Phi(x) - (-x) Phi(-x) = x (Phi(x) + Phi(-x)) = x
+    np.testing.assert_allclose(O.gelu(x) - O.gelu(-x), x, rtol=1e-12, atol=1e-15)
+    # the negative tail keeps its digits: x Phi(x) with Phi(-8.5) = 9.48e-18 from libm
+    import math
+    phi = 0.5 * math.erfc(8.5 / math.sqrt(2.0))
+    assert 9.47e-18 < phi < 9.49e-18
+    assert abs(O.gelu(np.array([-8.5]))[0] / (-8.5 * phi) - 1) < 1e-12
+    # backward: autograd of the library routine, and gelu'(x) + gelu'(-x) = 1
+    xt = torch.from_numpy(x).requires_grad_(True)
+    g = rng.standard_normal(x.size)
+    F.gelu(xt).backward(torch.from_numpy(g))
+    np.testing.assert_allclose(O.gelu_backward(g, x), xt.grad.numpy(), rtol=1e-11, atol=1e-14)
+    one = np.ones_like(x)
+    np.testing.assert_allclose(O.gelu_backward(one, x) + O.gelu_backward(one, -x), one,
+                               rtol=1e-12)
+    assert O.gelu_backward(np.array([1.0]), np.array([0.0]))[0] == 0.5
