@@ -21,7 +21,7 @@ struct GemmArgs {
   int in_feat;
   int out_feat;
   int n_expert;
-  int tile;             // 0 = choose the tile shape automatically, 1..3 = force one
+  int tile;             // 0 = choose the tile shape automatically, 1..4 = force one
 };
 
 // Virtual row-tile index space of the scalar kernel: expert e owns the tiles

@@ -23,13 +23,16 @@
 // descriptor's num_records and arrive as zeros, so there are no edge kernels
 // and no branches in the load path.
 //
-// NS (4) LDS stages of BK (32) values of K: two K-slices are always in flight
-// while one feeds the MFMAs; one barrier per slice.
+// Two pipelines: four LDS stages of 32 values of K (two K-slices in flight while
+// one feeds the MFMAs, one barrier per slice), or two stages of 64 values with
+// the barrier in front of the last K step (whole 128-byte lines for
+// K-contiguous operands).
 //
 // The rows of an expert are cut into BM-row tiles plus, for a remainder of at
 // most BM / 2 rows, one 64- or 128-row tile that costs a fraction of a BM tile,
-// so a few rows past a multiple of BM do not cost a whole tile.  Tiles are dealt to the
-// workgroups in an XCD-aware patch order.
+// so a few rows past a multiple of BM do not cost a whole tile; a last column
+// tile (or last row tile of dW) that is at most half full runs as a half-size
+// tile.  Tiles are dealt to the workgroups in an XCD-aware patch order.
 //
 // Operand roles follow cuda/parallel_linear.cuh:69-87,124-147 of the
 // reference; the per-expert cuBLAS loop there becomes a tile index space.
@@ -911,8 +914,8 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
 // round is really 256 wide), a tile costs a fixed prologue/epilogue
 // plus a per-K-slice time that depends on its shape (measured microseconds).
 // The shape with the least estimated time wins; `g.tile` overrides the choice
-// for tuning (1..3 = the three shapes, 4 = 256x256 with two stages of 64).  Ragged experts add at most one partial tile each, which
-// the estimate ignores.
+// for tuning (1..3 = the three shapes, 4 = 256x256 with two stages of 64).
+// Ragged experts add at most one partial tile each, which the estimate ignores.
 template <int MODE>
 static int pick_tile(const GemmArgs& g) {
   if (g.tile >= 1 && g.tile <= 4) return g.tile;
