@@ -144,6 +144,32 @@ def step(layer, x, dy):
     return out
 
 
+def graph_replay(layer, x, dy, cfg, steps):
+    """The same step captured once in a HIP graph and replayed `steps` times: the
+    layer enqueues without reading anything back, so the capture is legal and the
+    replay shows the step without its host-side launch cost."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(layer, x, dy)
+    torch.cuda.current_stream().wait_stream(side)
+    for p in layer.parameters():
+        p.grad = None
+    x.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        layer(x).backward(dy)
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"ms_per_step": round(ms, 4), "tokens_per_s": round(cfg["T"] / (ms * 1e-3), 1)}
+
+
 # ---------------------------------------------------------------- accounting
 def kernel_work(cfg: dict, n_valid: int):
     """Algorithmic FLOPs / bytes of ONE launch of each op on this workload."""
@@ -218,6 +244,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="cfg2", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the same steps replayed from one HIP graph (extra field)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures ONE GPU: this build has no multi-GPU path "
@@ -330,6 +358,8 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    if args.graph:
+        result["hip_graph"] = graph_replay(layer, x, dy, cfg, args.steps)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg, layer, x.detach())
     else:

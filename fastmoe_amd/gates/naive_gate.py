@@ -19,8 +19,9 @@ class NaiveGate(BaseGate):
     def forward(self, inp, return_all_scores=False):
         logits = self.gate(inp)
         top_idx, score = topk_softmax(logits, self.top_k)
-        # a zero loss so training loops can always call get_loss()
-        self.set_loss(torch.zeros(1, requires_grad=True).to(inp.device))
+        # a zero loss so training loops can always call get_loss(); created on the
+        # device (no host-to-device copy, so the forward can sit in a HIP graph)
+        self.set_loss(torch.zeros(1, device=inp.device, requires_grad=True))
         if return_all_scores:
             return top_idx, score, logits
         return top_idx, score
