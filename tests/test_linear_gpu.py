@@ -145,9 +145,9 @@ def test_errors_are_runtime_errors():
                                torch.zeros(2, dtype=torch.int32, device="cuda"))
 
 
-@pytest.mark.parametrize("cfg", ["cfg2", "cfg5"])
+@pytest.mark.parametrize("cfg", ["cfg2", "cfg4", "cfg5"])
 def test_full_size_gemm_properties(cfg):
-    """Full-size grouped GEMMs (the balanced and the fine-grained workload)
+    """Full-size grouped GEMMs (the balanced, the largest and the fine-grained workload)
     checked through properties that do not need a CPU evaluation: agreement with fp32 matmul of sampled rows, exact zeros
     for empty experts, and linearity in the input."""
     from fastmoe_amd import fmoe_cuda
@@ -155,6 +155,10 @@ def test_full_size_gemm_properties(cfg):
     if cfg == "cfg2":
         e, d, h, n = 16, 1024, 4096, 16384
         counts = torch.full((e,), n // e, dtype=torch.int64)
+    elif cfg == "cfg4":
+        e, d, h, n = 8, 4096, 14336, 32768
+        g = torch.Generator().manual_seed(4)
+        counts = torch.bincount(torch.randint(0, e, (n,), generator=g), minlength=e)
     else:
         e, d, h, n = 128, 2048, 1408, 65536
         g = torch.Generator().manual_seed(0)
@@ -188,3 +192,48 @@ def test_full_size_gemm_properties(cfg):
         assert max_rel_err(dx[rows], dy[rows].float() @ w[ex].float()) <= 2e-2
     for ex in np.flatnonzero(counts.numpy() == 0):
         assert not dw[ex].any().item() and not db[ex].any().item()
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_ragged_shapes_against_torch(seed):
+    """Random expert counts, row counts (empty experts included) and feature
+    sizes through the automatic kernel choice, against per-expert float32
+    matmuls of the same rounded operands on the GPU."""
+    from fastmoe_amd import fmoe_cuda
+
+    rng = np.random.default_rng(1000 + seed)
+    dt = [torch.bfloat16, torch.float16, torch.float32][seed % 3]
+    step = 4 if dt == torch.float32 else 8
+    e = int(rng.integers(1, 40))
+    in_f = int(rng.integers(1, 90)) * step
+    out_f = int(rng.integers(1, 90)) * step
+    if seed % 4 == 0:                      # a last column tile at most half full
+        out_f = 256 * int(rng.integers(1, 4)) + step * int(rng.integers(1, 16))
+    counts = rng.integers(0, 700, e) * (rng.random(e) < 0.8)
+    if seed % 5 == 0:
+        counts[rng.integers(0, e)] += 2048     # one expert with many full tiles
+    counts = torch.from_numpy(counts.astype(np.int64))
+    n = int(counts.sum())
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n + 2, in_f, generator=g).to(dt).cuda()
+    w = (torch.randn(e, out_f, in_f, generator=g) * 0.2).to(dt).cuda()
+    b = torch.randn(e, out_f, generator=g).to(dt).cuda()
+    dy = torch.randn(n + 2, out_f, generator=g).to(dt).cuda()
+    y = fmoe_cuda.linear_forward(x, counts, w, b)
+    dx, dw, db = fmoe_cuda.linear_backward(dy, x, counts, w, b)
+    tol = 2e-2 if dt == torch.bfloat16 else (4e-3 if dt == torch.float16 else 1e-4)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        off = 0
+        for ex in range(e):
+            c = int(counts[ex])
+            xs, ds, wf = x[off:off + c].float(), dy[off:off + c].float(), w[ex].float()
+            if c:
+                assert max_rel_err(y[off:off + c], xs @ wf.t() + b[ex].float()) <= tol
+                assert max_rel_err(dx[off:off + c], ds @ wf) <= tol
+            assert max_rel_err(dw[ex], ds.t() @ xs) <= tol
+            assert max_rel_err(db[ex], ds.sum(0)) <= tol
+            off += c
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
