@@ -16,6 +16,7 @@ namespace fmoe {
 constexpr int kGateThreads = 256;
 constexpr int kGateLanes = 8;                       // lanes per token
 constexpr int kGateTokens = kGateThreads / kGateLanes;
+constexpr int kGateChunk = 8;                       // logits a lane loads before it sorts them
 
 template <typename A>
 __device__ __forceinline__ bool better(A v, int e, A w, int f) {
@@ -40,19 +41,31 @@ __global__ __launch_bounds__(kGateThreads) void topk_softmax_fwd_kernel(
   }
   if (live) {
     const T* row = logits + t * n_expert;
-    for (int e = g; e < n_expert; e += kGateLanes) {
-      acc_t v = Elem<T>::to_acc(row[e]);
-      int ve = e;
-      // insertion into the sorted list: the displaced entry moves down
+    // kGateChunk loads in flight, then their insertions: one memory round trip
+    // per chunk instead of one per logit
+    for (int e0 = g; e0 < n_expert; e0 += kGateLanes * kGateChunk) {
+      T raw[kGateChunk];
 #pragma unroll
-      for (int j = 0; j < KMAX; ++j) {
-        if (better(v, ve, val[j], id[j])) {
-          const acc_t tv = val[j];
-          const int te = id[j];
-          val[j] = v;
-          id[j] = ve;
-          v = tv;
-          ve = te;
+      for (int u = 0; u < kGateChunk; ++u) {
+        const int e = e0 + u * kGateLanes;
+        if (e < n_expert) raw[u] = row[e];
+      }
+#pragma unroll
+      for (int u = 0; u < kGateChunk; ++u) {
+        int ve = e0 + u * kGateLanes;
+        if (ve >= n_expert) break;
+        acc_t v = Elem<T>::to_acc(raw[u]);
+        // insertion into the sorted list: the displaced entry moves down
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j) {
+          if (better(v, ve, val[j], id[j])) {
+            const acc_t tv = val[j];
+            const int te = id[j];
+            val[j] = v;
+            id[j] = ve;
+            v = tv;
+            ve = te;
+          }
         }
       }
     }
