@@ -281,6 +281,8 @@ def main():
             out[name] = {
                 "launches_per_step": len(ts) / n_steps,
                 "avg_us": round(avg_ms * 1e3, 2),
+                "median_us": round(sorted(ts)[len(ts) // 2] * 1e3, 2),
+                "min_us": round(min(ts) * 1e3, 2),
                 "total_ms_per_step": round(sum(ts) / n_steps, 4),
                 ("tflops" if kind == "flop" else "gbps"):
                     round(rate / (1e12 if kind == "flop" else 1e9), 2),
