@@ -225,7 +225,13 @@ def cpu_baseline(cfg: dict, layer, x, target_seconds: float = 15.0):
     run(probe)                                   # warm-up (thread pool, allocator)
     t_probe = run(probe)
     S = int(min(T, max(probe, probe * target_seconds / 3.0 / max(t_probe, 1e-6))))
-    times = [run(S) for _ in range(3)]
+    t_first = run(S)
+    # the small probe overstates the per-token cost (per-expert overheads):
+    # rescale once from the first full-size run
+    if t_first < target_seconds / 6.0 and S < T:
+        S = int(min(T, S * target_seconds / 3.0 / max(t_first, 1e-6)))
+        t_first = run(S)
+    times = [t_first] + [run(S) for _ in range(2)]
     best = min(times)
     return {
         "value": S / best,
