@@ -1,6 +1,5 @@
 """The C-ABI library loads and exports exactly what include/fmoe_hip.h declares
 (no compute calls: this runs without a GPU)."""
-import ctypes
 import os
 import re
 

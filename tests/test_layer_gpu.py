@@ -3,7 +3,6 @@ test oracle (tests/moe.py:30-49), mirroring tests/test_numerical.py,
 tests/test_zero.py and the invariants of tests/test_gates.py."""
 import math
 
-import numpy as np
 import pytest
 import torch
 import torch.nn.functional as F
