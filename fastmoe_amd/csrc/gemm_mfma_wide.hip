@@ -11,11 +11,12 @@
 // bf16 kernel (gemm.h); the row tiles of an expert are found as in the scalar
 // kernel (virtual_row_tiles).
 //
-// LDS holds both operands K-major, [k][row], so the MFMA operand of a lane
-// (one value: row = lane % block, k = lane / block) is a conflict-free 4- or
-// 8-byte read.  Operands that are K-contiguous in memory (X and W in FWD, dY in
-// DGRAD) are transposed on the way in (4-element packs read along K, written
-// as 4 single values); the others are copied pack by pack.
+// Both operand layouts are copied into LDS as they come, pack by pack: operands
+// whose rows are contiguous in memory (W in DGRAD, both in WGRAD) as [k][row],
+// K-contiguous ones (X and W in FWD, dY in DGRAD) as [row][k].  The MFMA takes
+// one value of K per lane; the lanes pick their values so that a [row][k]
+// operand is read as one 4-element pack per four MFMA rounds and a [k][row]
+// operand as single values of the same K (see the K loop).
 #include "gemm.h"
 
 namespace fmoe {
@@ -57,16 +58,29 @@ template <> struct WideMma<double> {
   }
 };
 
+// Elements of one operand slice in LDS: [k][row] rows of kWideTile + kPad, or
+// [row][k] rows of kBK values + 16 bytes (whichever is larger, so that either
+// layout fits).
+template <typename F>
+constexpr int wide_operand_elems() {
+  constexpr int by_k = WideMma<F>::kBK * (kWideTile + WideMma<F>::kPad);
+  constexpr int by_row = kWideTile * (WideMma<F>::kBK + 16 / (int)sizeof(F));
+  return by_k > by_row ? by_k : by_row;
+}
 template <typename F>
 constexpr size_t wide_lds_bytes() {
-  return (size_t)2 * 2 * WideMma<F>::kBK * (kWideTile + WideMma<F>::kPad) * sizeof(F);
+  return (size_t)2 * 2 * wide_operand_elems<F>() * sizeof(F);
 }
 
 template <typename F, int MODE>
 __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_kernel(GemmArgs g) {
   using Mma = WideMma<F>;
   constexpr int BK = Mma::kBK, BLK = Mma::kBlk, LD = kWideTile + Mma::kPad;
-  constexpr int kOperand = BK * LD;           // elements of one operand slice
+  constexpr int LDK = BK + 16 / (int)sizeof(F);   // row length of a [row][k] image
+  constexpr int kOperand = wide_operand_elems<F>();
+  // K values one MFMA round of 4 covers: a lane holds 4 consecutive ones
+  constexpr int kGroup = 4 * (64 / BLK);
+  static_assert(BK % kGroup == 0, "slices are whole groups of K");
   constexpr int kVecs = BK * kWideTile / 4 / kWideThreads;   // packs per thread and operand
   constexpr int TB = 64 / BLK;                // MFMA blocks per wave and direction
   constexpr bool A_KC = MODE != GEMM_WGRAD;   // operand is K-contiguous in memory
@@ -156,8 +170,7 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
       const int idx = tid + u * kWideThreads;
       if (kc) {
         const int row = idx / (BK / 4), kq = idx % (BK / 4);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) dst[(4 * kq + c) * LD + row] = r[u][c];
+        *reinterpret_cast<Vec4*>(dst + row * LDK + 4 * kq) = r[u];
       } else {
         const int k = idx / (kWideTile / 4), q = idx % (kWideTile / 4);
         *reinterpret_cast<Vec4*>(dst + k * LD + 4 * q) = r[u];
@@ -196,20 +209,38 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
       fetch(ra, a_base, lda, a_kc{}, m_valid, (kt + 1) * BK);
       fetch(rb, b_base, ldb, b_kc{}, n_valid, (kt + 1) * BK);
     }
+    // The MFMA wants, per lane, one value of K out of kStep; WHICH value of the
+    // slice that is only has to agree between the two operands.  Lane group lk
+    // takes k = 4 lk + c in round c of a group of kGroup values, so that a
+    // [row][k] operand is read as one 4-element pack per 4 rounds.
 #pragma unroll
-    for (int kk = 0; kk < BK / Mma::kStep; ++kk) {
-      F a[TB], b[TB];
+    for (int s = 0; s < BK / kGroup; ++s) {
+      Vec4 a[TB], b[TB];
+      const int k4 = s * kGroup + 4 * lk;
 #pragma unroll
-      for (int i = 0; i < TB; ++i)
-        a[i] = as[(kk * Mma::kStep + lk) * LD + wave_m * 64 + i * BLK + lr];
+      for (int i = 0; i < TB; ++i) {
+        const int row = wave_m * 64 + i * BLK + lr;
+        if (A_KC) a[i] = *reinterpret_cast<const Vec4*>(as + row * LDK + k4);
+        else
 #pragma unroll
-      for (int j = 0; j < TB; ++j)
-        b[j] = bs[(kk * Mma::kStep + lk) * LD + wave_n * 64 + j * BLK + lr];
+          for (int c = 0; c < 4; ++c) a[i][c] = as[(k4 + c) * LD + row];
+      }
 #pragma unroll
-      for (int i = 0; i < TB; ++i)
+      for (int j = 0; j < TB; ++j) {
+        const int row = wave_n * 64 + j * BLK + lr;
+        if (B_KC) b[j] = *reinterpret_cast<const Vec4*>(bs + row * LDK + k4);
+        else
 #pragma unroll
-        for (int j = 0; j < TB; ++j)
-          acc[i][j] = Mma::kSwap ? Mma::run(b[j], a[i], acc[i][j]) : Mma::run(a[i], b[j], acc[i][j]);
+          for (int c = 0; c < 4; ++c) b[j][c] = bs[(k4 + c) * LD + row];
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int i = 0; i < TB; ++i)
+#pragma unroll
+          for (int j = 0; j < TB; ++j)
+            acc[i][j] = Mma::kSwap ? Mma::run(b[j][c], a[i][c], acc[i][j])
+                                   : Mma::run(a[i][c], b[j][c], acc[i][j]);
     }
     if (more) {
       // the other stage was last read in iteration kt - 1, which every wave
