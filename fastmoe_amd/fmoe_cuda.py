@@ -486,6 +486,5 @@ def gelu_bwd(dy: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
 def set_gemm_path(path: int) -> None:
     """0 = matrix-core kernel where the shape allows (tile shape chosen by the
     library), 1 = scalar kernel only, 2..5 = matrix-core kernel with bf16/f16
-    tile configuration 1..4 forced; for f32/f64 any of 2..5 selects their
-    matrix-core kernel at every problem size (for tests and tuning)."""
+    tile configuration 1..4 forced (for tests and tuning)."""
     _lib.check(_L.fmoe_set_gemm_path(path), "set_gemm_path")

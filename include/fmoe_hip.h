@@ -194,8 +194,8 @@ int fmoe_scatter_reduce(const void* dbuf, const int32_t* inv, void* dx,
  *   y [n_rows, out_feat]; seg_off is a DEVICE int32[E+1].
  * Rows at or beyond seg_off[E] are not written.  Empty experts cost nothing.
  * bf16/f16: MFMA with fp32 accumulation.  f32/f64: accumulation in the same
- * type, on the matrix cores when both feature sizes are multiples of 4 and the
- * problem fills the chip, else in a scalar kernel.
+ * type, on the matrix cores when both feature sizes are multiples of 4, else in
+ * a scalar kernel.
  * Replaces fmoe_cuda.linear_forward: cuda/fmoe_cuda.cpp:48-53,
  * cuda/parallel_linear.cu:5-50, cuda/parallel_linear.cuh:55-89.
  */
@@ -273,8 +273,7 @@ int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, int dtype,
  * Selects the grouped-GEMM kernel family: 0 = automatic (MFMA where the shape
  * allows, tile shape from the library's cost model), 1 = force the scalar
  * kernel, 2..5 = MFMA with bf16/f16 tile configuration 1..4 forced (256x256,
- * 128x256, 128x128, 256x256 with K slices of 64; f32/f64 have one tile shape,
- * which any of 2..5 selects at every problem size).  A testing and tuning aid
+ * 128x256, 128x128, 256x256 with K slices of 64; f32/f64 have one tile shape).  A testing and tuning aid
  * with no counterpart in the reference; process-wide, not thread-safe.
  */
 int fmoe_set_gemm_path(int path);

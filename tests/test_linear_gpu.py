@@ -97,14 +97,13 @@ def test_matrix_core_forced_tile(dt, tile, counts, in_f, out_f):
 @pytest.mark.parametrize("with_bias", [True, False])
 @pytest.mark.parametrize("counts,in_f,out_f", SHAPES + FORCED)
 def test_matrix_core_full_precision(dt, with_bias, counts, in_f, out_f):
-    # forcing a tile configuration sends f32 / f64 to their matrix-core kernel at
-    # any size (shapes that are not multiples of 4 still take the scalar kernel)
-    _run(counts, in_f, out_f, DTYPES[dt], with_bias, path=2, extra_rows=3)
+    # f32 / f64 on their matrix-core kernel (shapes that are not multiples of 4
+    # still take the scalar kernel)
+    _run(counts, in_f, out_f, DTYPES[dt], with_bias, path=0, extra_rows=3)
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
-def test_matrix_core_full_precision_chosen_by_size(dt):
-    # large enough for the library to pick the matrix cores by itself
+def test_matrix_core_full_precision_many_tiles(dt):
     _run([2100, 0, 1500, 4000, 37, 900], 256, 512, DTYPES[dt], True, path=0, extra_rows=9)
 
 
