@@ -20,6 +20,12 @@ CASES = [  # tokens, experts, top_k
     (19, 100, 16),      # largest supported top_k
     (7, 4096, 3),
     (1000, 7, 7),       # every expert chosen
+    (50, 256, 8),       # up to 512 experts: logits held in registers (8 per lane here)
+    (33, 300, 4),       # 32 lanes per token, ragged last register
+    (20, 512, 16),
+    (40, 17, 3),
+    (40, 40, 5),
+    (9, 513, 2),        # above 512: sorted lists over 32 lanes
 ]
 SCORE_TOL = {"f64": 1e-12, "f32": 2e-6, "f16": 2e-3, "bf16": 1.6e-2}
 
@@ -63,6 +69,20 @@ def test_ties_and_minus_infinity():
     idx, score = fmoe_cuda.topk_softmax_fwd(lt.cuda(), 2)
     assert idx.cpu().tolist() == [[1, 2], [0, 1], [2, 4]]
     want = O.topk_softmax(lt.double().numpy(), 2)[1]
+    assert np.abs(score.double().cpu().numpy() - want).max() <= 1e-6
+
+
+def test_ties_and_minus_infinity_in_a_wide_expert_set():
+    from fastmoe_amd import fmoe_cuda
+
+    e = 70
+    lt = torch.full((3, e), float("-inf"))
+    lt[0, [5, 40, 69]] = torch.tensor([2.0, 2.0, 2.0])       # three-way tie
+    lt[1, 33] = 1.0                                           # one finite logit, k = 3
+    lt[2] = 0.5                                               # all equal
+    idx, score = fmoe_cuda.topk_softmax_fwd(lt.cuda(), 3)
+    assert idx.cpu().tolist() == [[5, 40, 69], [33, 0, 1], [0, 1, 2]]
+    want = O.topk_softmax(lt.double().numpy(), 3)[1]
     assert np.abs(score.double().cpu().numpy() - want).max() <= 1e-6
 
 
