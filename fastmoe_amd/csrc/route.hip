@@ -63,6 +63,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_hist_global_kernel(
 }
 
 // --------------------------------------------------------------------- scan
+constexpr int kScanChunk = 8;   // per-block counters a thread loads before it sums them
 template <int MODE>
 __global__ __launch_bounds__(kScanThreads) void route_scan_kernel(
     int32_t* __restrict__ block_hist, int n_blocks, int n_expert,
@@ -72,13 +73,20 @@ __global__ __launch_bounds__(kScanThreads) void route_scan_kernel(
   int32_t* cnt = lds_scan;                  // [E]
   int32_t* off = lds_scan + n_expert;       // [E+1]
   // exclusive scan over the blocks, one expert per thread
+  // (kScanChunk loads in flight at a time: one memory round trip per chunk
+  // instead of one per block)
   for (int e = threadIdx.x; e < n_expert; e += kScanThreads) {
     int32_t run = 0;
-    for (int b = 0; b < n_blocks; ++b) {
-      const int64_t at = (int64_t)b * n_expert + e;
-      const int32_t v = block_hist[at];
-      block_hist[at] = run;
-      run += v;
+    for (int b0 = 0; b0 < n_blocks; b0 += kScanChunk) {
+      int32_t v[kScanChunk];
+#pragma unroll
+      for (int u = 0; u < kScanChunk; ++u)
+        v[u] = b0 + u < n_blocks ? block_hist[(int64_t)(b0 + u) * n_expert + e] : 0;
+#pragma unroll
+      for (int u = 0; u < kScanChunk; ++u) {
+        if (b0 + u < n_blocks) block_hist[(int64_t)(b0 + u) * n_expert + e] = run;
+        run += v[u];
+      }
     }
     cnt[e] = run;
   }
