@@ -5,9 +5,10 @@
 //
 // These MFMAs run at 1/16 (f32) and 1/32 (f64) of the bf16 rate, so one K slice
 // of a 128x128 tile keeps the matrix cores busy for microseconds and a plain
-// design is enough: global -> registers -> LDS with two LDS stages, one barrier
-// per slice, two blocks per CU so that one block's barrier and LDS writes hide
-// behind the other's MFMAs.  Operand roles and the ragged rows are those of the
+// design is enough: global -> registers -> LDS with two LDS stages of 16 values
+// of K, one barrier per slice, and several blocks per CU (three or four for
+// f32, two for f64) so that one block's barrier and LDS writes hide behind the
+// others' MFMAs.  Operand roles and the ragged rows are those of the
 // bf16 kernel (gemm.h); the row tiles of an expert are found as in the scalar
 // kernel (virtual_row_tiles).
 //
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
 template <typename F, int MODE>
 int launch_wide_mode(const GemmArgs& g, hipStream_t s) {
   constexpr size_t lds = wide_lds_bytes<F>();
-  static_assert(2 * (lds + 64) <= 160 * 1024, "two blocks per gfx950 CU");
+  static_assert(2 * (lds + 64) <= 160 * 1024, "at least two blocks per gfx950 CU");
   auto kern = gemm_wide_kernel<F, MODE>;
   static bool configured = false;  // attribute is per function, set once
   if (!configured) {
