@@ -6,8 +6,8 @@
 // These MFMAs run at 1/16 (f32) and 1/32 (f64) of the bf16 rate, so one K slice
 // of a 128x128 tile keeps the matrix cores busy for microseconds and a plain
 // design is enough: global -> registers -> LDS with two LDS stages of 16 values
-// of K, one barrier per slice, and several blocks per CU (three or four for
-// f32, two for f64) so that one block's barrier and LDS writes hide behind the
+// of K, one barrier per slice, and several blocks per CU (four for f32: their
+// stages fill the 160 KB of LDS exactly; two for f64) so that one block's barrier and LDS writes hide behind the
 // others' MFMAs.  Operand roles and the ragged rows are those of the
 // bf16 kernel (gemm.h); the row tiles of an expert are found as in the scalar
 // kernel (virtual_row_tiles).
@@ -89,7 +89,6 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
   using Vec4 = typename Mma::vec_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   F* smem = reinterpret_cast<F*>(smem_raw);   // [stage][A | B][k][row]
-  __shared__ int s_expert;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wave_m = wave >> 1, wave_n = wave & 1;
@@ -99,18 +98,15 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
     e = blockIdx.z;
     m_tile = blockIdx.y;
   } else {
-    // the expert that owns virtual row tile blockIdx.y
+    // the expert that owns virtual row tile blockIdx.y (every thread searches:
+    // the loads are uniform, and LDS is left to the operand stages)
     const int v = blockIdx.y;
-    if (tid == 0) {
-      int lo = 0, hi = g.n_expert - 1;
-      while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (g.seg_off[mid] / kWideTile + mid <= v) lo = mid; else hi = mid - 1;
-      }
-      s_expert = lo;
+    int lo = 0, hi = g.n_expert - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (g.seg_off[mid] / kWideTile + mid <= v) lo = mid; else hi = mid - 1;
     }
-    __syncthreads();
-    e = s_expert;
+    e = lo;
     m_tile = v - (g.seg_off[e] / kWideTile + e);
   }
   const int64_t row0 = g.seg_off[e];
@@ -296,7 +292,7 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
 template <typename F, int MODE>
 int launch_wide_mode(const GemmArgs& g, hipStream_t s) {
   constexpr size_t lds = wide_lds_bytes<F>();
-  static_assert(2 * (lds + 64) <= 160 * 1024, "at least two blocks per gfx950 CU");
+  static_assert(2 * lds <= 160 * 1024, "at least two blocks per gfx950 CU");
   auto kern = gemm_wide_kernel<F, MODE>;
   static bool configured = false;  // attribute is per function, set once
   if (!configured) {
