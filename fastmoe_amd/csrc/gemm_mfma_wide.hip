@@ -32,7 +32,6 @@ constexpr int kWideThreads = 256;  // 2 x 2 waves of 64 x 64
 template <typename F> struct WideMma;
 template <> struct WideMma<float> {
   static constexpr int kBlk = 32;   // rows / columns of one MFMA block
-  static constexpr int kStep = 2;   // values of K per MFMA
   static constexpr int kAcc = 16;   // accumulators per lane and block
   static constexpr int kBK = 16;    // values of K per LDS slice
   static constexpr int kPad = 4;    // row padding of the LDS image, in elements
@@ -46,7 +45,6 @@ template <> struct WideMma<float> {
 };
 template <> struct WideMma<double> {
   static constexpr int kBlk = 16;
-  static constexpr int kStep = 4;
   static constexpr int kAcc = 4;
   static constexpr int kBK = 16;
   static constexpr int kPad = 2;
