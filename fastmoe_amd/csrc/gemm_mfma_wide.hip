@@ -204,7 +204,7 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
       fetch(ra, a_base, lda, a_kc{}, m_valid, (kt + 1) * BK);
       fetch(rb, b_base, ldb, b_kc{}, n_valid, (kt + 1) * BK);
     }
-    // The MFMA wants, per lane, one value of K out of kStep; WHICH value of the
+    // The MFMA wants, per lane, one value of K out of 64 / BLK; WHICH value of the
     // slice that is only has to agree between the two operands.  Lane group lk
     // takes k = 4 lk + c in round c of a group of kGroup values, so that a
     // [row][k] operand is read as one 4-element pack per 4 rounds.
