@@ -8,6 +8,15 @@ from .. import fmoe_cuda as fmoe_native
 from .naive_gate import NaiveGate
 
 
+def _histogram(idx, n_expert):
+    r"""Entries of `idx` per expert (`-1` skipped), int32 on the device, by the
+    library's histogram kernel: nothing is read back to the host, which keeps
+    the gate inside a HIP graph."""
+    count = torch.zeros(n_expert, dtype=torch.int32, device=idx.device)
+    fmoe_native.expert_count(idx.contiguous(), count)
+    return count
+
+
 class GShardGate(NaiveGate):
     r"""Top-2 gate with a load-balance loss, a per-expert capacity of
     `ceil(rate * tokens) * 2 // experts` slots (rate = `capacity[0]` in
@@ -25,7 +34,7 @@ class GShardGate(NaiveGate):
         topk_idx, topk_val, logits = super().forward(x, return_all_scores=True)
         n_tok = logits.shape[0]
         top1 = topk_idx.view(-1, self.top_k)[:, 0]
-        frac = torch.bincount(top1, minlength=self.tot_expert).to(torch.float) / n_tok
+        frac = _histogram(top1, self.tot_expert).to(torch.float) / n_tok
         prob = F.softmax(logits, dim=1).mean(dim=0)
         self.set_loss(torch.mean(frac * prob) * (self.num_expert ** 2))
 

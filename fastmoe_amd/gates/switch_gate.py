@@ -4,6 +4,7 @@ import math
 import torch
 import torch.nn.functional as F
 
+from .gshard_gate import _histogram
 from .naive_gate import NaiveGate
 from .utils import limit_by_capacity
 
@@ -34,8 +35,12 @@ class SwitchGate(NaiveGate):
         _lec, _gec, top1_idx = limit_by_capacity(top1_idx, self.num_expert,
                                                  self.world_size, cap)
 
-        kept = top1_idx[top1_idx > -1]
-        frac = torch.bincount(kept, minlength=self.tot_expert).to(torch.float) / kept.numel()
-        prob = score.sum(dim=0) / kept.numel()
+        # per-expert counts of the slots that survived, and their total, stay on
+        # the device (fmoe/gates/switch_gate.py:49-57 indexes with a mask, which
+        # reads the number of survivors back to the host)
+        count = _histogram(top1_idx, self.tot_expert).to(torch.float)
+        n_kept = count.sum()
+        frac = count / n_kept
+        prob = score.sum(dim=0) / n_kept
         self.set_loss((frac * prob).sum() * self.tot_expert)
         return top1_idx, top1_score

@@ -215,12 +215,13 @@ def test_zero_token_experts_and_mask():
 def test_gshard_gate_invariants(n_expert, cap):
     """tests/test_gates.py:31-56: per-expert load <= ceil(cap * batch), kept
     scores equal the plain top-2 softmax."""
-    from fastmoe_amd.gates import GShardGate
+    from fastmoe_amd.gates import GShardGate, NaiveGate
 
     torch.manual_seed(0)
     gate = GShardGate(1024, n_expert, 1, capacity=(cap, cap)).cuda()
     x = torch.rand(16, 1024).cuda()
     idx, val = gate(x)
+    loss = gate.get_loss()
     counts = torch.bincount(idx[idx >= 0].view(-1), minlength=n_expert)
     assert counts.max().item() <= math.ceil(cap * 16)
     logits = gate.gate(x)
@@ -228,6 +229,11 @@ def test_gshard_gate_invariants(n_expert, cap):
     ref = F.softmax(tv, dim=-1)
     keep = idx != -1
     assert torch.equal(val[keep], ref[keep])
+    # the balance loss (fmoe/gates/gshard_gate.py:26-33) from torch.bincount
+    _i, _v, lg = NaiveGate.forward(gate, x, return_all_scores=True)
+    frac = torch.bincount(_i[:, 0], minlength=n_expert).float() / 16
+    want = torch.mean(frac * F.softmax(lg, dim=1).mean(dim=0)) * n_expert ** 2
+    assert abs(loss.item() - want.item()) <= 1e-6 * max(1.0, abs(want.item()))
 
 
 @pytest.mark.parametrize("n_expert,cap", [(1, 0.1), (16, 0.8)])
@@ -245,7 +251,11 @@ def test_switch_gate_invariants(n_expert, cap):
     keep = (idx != -1).view(-1)
     rows = torch.nonzero(keep).view(-1)
     assert torch.equal(val.view(-1)[rows], score[rows, idx.view(-1)[rows]])
-    assert gate.get_loss() is not None
+    # the balance loss (fmoe/gates/switch_gate.py:49-57) from torch.bincount
+    kept = idx[idx > -1]
+    frac = torch.bincount(kept, minlength=n_expert).float() / kept.numel()
+    want = (frac * (score.sum(dim=0) / kept.numel())).sum() * n_expert
+    assert abs(gate.get_loss().item() - want.item()) <= 1e-5 * max(1.0, abs(want.item()))
 
 
 def test_dropped_slots_flow_through_the_layer():
