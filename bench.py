@@ -58,6 +58,8 @@ PEAK = {"hbm": 8.0e12, "bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 MEASURED_TRAFFIC = {
     ("cfg2", "grouped_linear_bwd"): (273.9 + 208.0) * 2 ** 20,
     ("cfg2", "grouped_linear_fwd"): (153.7 + 80.0) * 2 ** 20,
+    ("cfg5", "grouped_linear_bwd"): (1185.5 + 920.0) * 2 ** 20,
+    ("cfg5", "grouped_linear_fwd"): (808.7 + 216.0) * 2 ** 20,
 }
 
 
