@@ -188,6 +188,7 @@ def kernel_work(cfg: dict, n_valid: int):
         "grouped_linear_bias_grad": ("byte", n_valid * (d + h) / 2.0 * s),
         "route": ("byte", 8.0 * N + 8.0 * n_valid + 4.0 * N + 8.0 * N),
         "local_scatter": ("byte", 2.0 * n_valid * d * s + 8.0 * n_valid),
+        "scatter_tokens": ("byte", T * d * s + n_valid * d * s + 4.0 * N),
         "gather_combine_fwd": ("byte", n_valid * d * s + T * d * s + N * (4 + s)),
         "gather_combine_bwd": ("byte", T * d * s + 2.0 * n_valid * d * s + N * (4 + 2 * s)),
         "scatter_reduce": ("byte", n_valid * d * s + T * d * s + 4.0 * N),

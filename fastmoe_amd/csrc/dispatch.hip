@@ -246,6 +246,37 @@ __global__ __launch_bounds__(kDispThreads) void combine_bwd_kernel(
   }
 }
 
+// out[inv[t * k + j]] = inp[t] for every live slot of token t: the scatter in
+// token order.  A token row is read once and written k times, where the
+// row-ordered scatter reads it k times at k distant moments (with k = 8 most of
+// those reads miss L2).  One wave per token; lane j < k holds the row of slot j.
+template <typename V>
+__global__ __launch_bounds__(kDispThreads) void scatter_tokens_kernel(
+    const V* __restrict__ inp, const int32_t* __restrict__ inv, V* __restrict__ out,
+    int64_t n_tokens, int top_k, int64_t row_vecs) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t)blockIdx.x * kDispWaves + threadIdx.x / kWave;
+  const int64_t n_waves = (int64_t)gridDim.x * kDispWaves;
+  for (int64_t t = wave; t < n_tokens; t += n_waves) {
+    const int32_t my_r = lane < top_k ? inv[t * top_k + lane] : -1;
+    const V* s = inp + t * row_vecs;
+    for (int64_t c0 = lane; c0 < row_vecs; c0 += 4 * kWave) {
+      V a[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (c0 + u * kWave < row_vecs) a[u] = s[c0 + u * kWave];
+      for (int j = 0; j < top_k; ++j) {
+        const int32_t r = lane_value(my_r, j);
+        if (r < 0) continue;  // dropped slot (the same for the whole wave)
+        V* d = out + (int64_t)r * row_vecs;
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (c0 + u * kWave < row_vecs) d[c0 + u * kWave] = a[u];
+      }
+    }
+  }
+}
+
 // ----------------------------------------------------------------- host side
 static int grid_for_rows(int64_t rows) {
   int64_t blocks = (rows + kDispWaves - 1) / kDispWaves;
@@ -367,6 +398,47 @@ extern "C" int fmoe_local_scatter(const void* inp, const int64_t* idx, void* out
       break;
   }
   FMOE_LAUNCH_CHECK("local_scatter");
+  return FMOE_OK;
+}
+
+extern "C" int fmoe_scatter_tokens(const void* inp, const int32_t* inv, void* out,
+                                   int64_t n_tokens, int64_t top_k, int64_t d, int dtype,
+                                   void* stream) {
+  const int64_t es = (int64_t)dtype_size(dtype);
+  FMOE_REQUIRE(es != 0, FMOE_ERR_INVALID, "scatter_tokens: unknown dtype %d", dtype);
+  FMOE_REQUIRE(n_tokens >= 0 && d >= 0 && top_k >= 1, FMOE_ERR_INVALID,
+               "scatter_tokens: bad sizes tokens=%lld d=%lld top_k=%lld", (long long)n_tokens,
+               (long long)d, (long long)top_k);
+  FMOE_REQUIRE(top_k <= kWave, FMOE_ERR_UNSUPPORTED, "scatter_tokens: top_k %lld exceeds %d",
+               (long long)top_k, kWave);
+  if (n_tokens == 0 || d == 0) return FMOE_OK;
+  FMOE_REQUIRE(inp && inv && out, FMOE_ERR_INVALID, "scatter_tokens: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t row_bytes = d * es;
+  const int grid = grid_for_rows(n_tokens);
+  switch (copy_unit(inp, out, row_bytes)) {
+    case 16:
+      hipLaunchKernelGGL(scatter_tokens_kernel<uint4>, dim3(grid), dim3(kDispThreads), 0, s,
+                         (const uint4*)inp, inv, (uint4*)out, n_tokens, (int)top_k,
+                         row_bytes / 16);
+      break;
+    case 8:
+      hipLaunchKernelGGL(scatter_tokens_kernel<uint64_t>, dim3(grid), dim3(kDispThreads), 0, s,
+                         (const uint64_t*)inp, inv, (uint64_t*)out, n_tokens, (int)top_k,
+                         row_bytes / 8);
+      break;
+    case 4:
+      hipLaunchKernelGGL(scatter_tokens_kernel<uint32_t>, dim3(grid), dim3(kDispThreads), 0, s,
+                         (const uint32_t*)inp, inv, (uint32_t*)out, n_tokens, (int)top_k,
+                         row_bytes / 4);
+      break;
+    default:
+      hipLaunchKernelGGL(scatter_tokens_kernel<uint16_t>, dim3(grid), dim3(kDispThreads), 0, s,
+                         (const uint16_t*)inp, inv, (uint16_t*)out, n_tokens, (int)top_k,
+                         row_bytes / 2);
+      break;
+  }
+  FMOE_LAUNCH_CHECK("scatter_tokens");
   return FMOE_OK;
 }
 

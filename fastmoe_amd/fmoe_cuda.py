@@ -248,6 +248,23 @@ def local_scatter(inp: torch.Tensor, pos: torch.Tensor, idx_div: int = 1,
     return out
 
 
+def scatter_tokens(inp: torch.Tensor, inv: torch.Tensor, top_k: int) -> torch.Tensor:
+    """buf[inv[t * top_k + j]] = inp[t] for live slots: local_scatter in token
+    order (one read per token row).  Rows of buf no slot maps to are not written."""
+    _dev(inp, "inp")
+    _dev(inv, "inv", torch.int32)
+    _need(inp.dim() == 2, "inp must be [tokens, d]")
+    t, d = inp.shape
+    _need(inv.numel() == t * top_k, "inv must have tokens * top_k entries")
+    out = torch.empty((t * top_k, d), dtype=inp.dtype, device=inp.device)
+    with _launch(inp, "scatter_tokens"):
+        _lib.check(
+            _L.fmoe_scatter_tokens(inp.data_ptr(), inv.data_ptr(), out.data_ptr(), t, top_k, d,
+                                   _dt(inp, "inp"), _stream(inp)),
+            "scatter_tokens")
+    return out
+
+
 def local_gather(inp: torch.Tensor, pos: torch.Tensor, out_batch_size: int,
                  maybe_overlap: bool = True,
                  n_rows_dev: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -152,6 +152,10 @@ class FusedScatter(Function):
     @staticmethod
     def forward(ctx, inp, plan: RoutePlan):
         ctx.plan = plan
+        if 4 <= plan.top_k <= 64:
+            # token order: a row is read once for its k copies (measured: 62 vs 81 us
+            # at k = 8 on 8192 x 2048 bf16; at k = 2 the row order is the faster one)
+            return fmoe_cuda.scatter_tokens(inp.contiguous(), plan.inv, plan.top_k)
         return fmoe_cuda.local_scatter(inp.contiguous(), plan.pos, plan.top_k,
                                        plan.n_rows_dev)
 

@@ -144,6 +144,18 @@ int fmoe_local_scatter(const void* inp, const int64_t* idx, void* out,
                        const int32_t* n_rows_dev, int dtype, void* stream);
 
 /*
+ * out[inv[t * top_k + j]] = inp[t] for every slot with inv >= 0: the same rows
+ * as fmoe_local_scatter(inp, pos, ..., idx_div = top_k) writes, produced in
+ * token order from the inverse map of fmoe_route (a token row is read once for
+ * its top_k copies).  inp [n_tokens, d], out [>= live rows, d]; top_k <= 64.
+ * Replaces fmoe.functions._local_scatter (fmoe/functions.py:78-80) in
+ * MOEScatter.forward (functions.py:100-121) when the inverse map is at hand.
+ */
+int fmoe_scatter_tokens(const void* inp, const int32_t* inv, void* out,
+                        int64_t n_tokens, int64_t top_k, int64_t d, int dtype,
+                        void* stream);
+
+/*
  * overlap == 0: out = 0 [out_rows, d]; out[pos[r]] = inp[r]  (pos distinct).
  * overlap != 0: out[p] = sum over {r : pos[r] == p} inp[r]; f32/f64 only
  *               (device float atomics, summation order unspecified, as with

@@ -56,6 +56,9 @@ def test_scatter_and_gather_are_exact_copies(dt, n, k, e, d, drop):
     del full
     back = fmoe_cuda.local_gather(buf, pos_c, n * k, maybe_overlap=False)
     assert np.array_equal(_bits(back), O.local_gather(want, pos, n * k))
+    # the same rows written in token order from the inverse map
+    buf3 = fmoe_cuda.scatter_tokens(x.cuda(), torch.from_numpy(inv.astype(np.int32)).cuda(), k)
+    assert np.array_equal(_bits(buf3)[: pos.size], want)
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64", "bf16"])
