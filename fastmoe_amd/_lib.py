@@ -53,8 +53,9 @@ SIGNATURES = {
                                       c_int32, c_int, c_void_p]),
     "fmoe_scatter_tokens": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                     c_int, c_void_p]),
-    "fmoe_gelu_fwd": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
-    "fmoe_gelu_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "fmoe_gelu_fwd": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p]),
+    "fmoe_gelu_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int,
+                              c_void_p]),
     "fmoe_set_gemm_path": (c_int, [c_int]),
 }
 

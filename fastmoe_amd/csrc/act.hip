@@ -53,10 +53,22 @@ __global__ void gelu_table_kernel() {
   }
 }
 
+// Elements that need work: all n, or the first *n_rows_dev rows of row_len when
+// the caller knows that the rows behind them are dead (slots dropped by a
+// capacity limit leave such rows at the end of the expert-ordered buffers).
+__device__ __forceinline__ int64_t live_elems(int64_t n, const int32_t* n_rows_dev,
+                                              int64_t row_len) {
+  if (n_rows_dev == nullptr) return n;
+  const int64_t live = (int64_t)*n_rows_dev * row_len;
+  return live < n ? live : n;
+}
+
 // ---- 16-bit types: table in LDS ------------------------------------------
 // x, y: n_packs 16-byte packs of 8 elements.
 __global__ __launch_bounds__(kActThreads) void gelu_fwd_lut_kernel(
-    const uint4* __restrict__ x, uint4* __restrict__ y, int64_t n_packs, int which) {
+    const uint4* __restrict__ x, uint4* __restrict__ y, int64_t n_packs, int which,
+    const int32_t* __restrict__ n_rows_dev, int64_t row_packs) {
+  n_packs = live_elems(n_packs, n_rows_dev, row_packs);
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   uint16_t* lut = reinterpret_cast<uint16_t*>(lds_raw);
   {
@@ -87,7 +99,8 @@ __global__ __launch_bounds__(kActThreads) void gelu_fwd_lut_kernel(
 template <typename T>
 __global__ __launch_bounds__(kActThreads) void gelu_bwd_lut_kernel(
     const uint4* __restrict__ dy, const uint4* __restrict__ x, uint4* __restrict__ dx,
-    int64_t n_packs, int which) {
+    int64_t n_packs, int which, const int32_t* __restrict__ n_rows_dev, int64_t row_packs) {
+  n_packs = live_elems(n_packs, n_rows_dev, row_packs);
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   float* lut = reinterpret_cast<float*>(lds_raw);
   {
@@ -152,14 +165,20 @@ __device__ __forceinline__ float gelu_grad_direct(float x) {
 __device__ __forceinline__ double gelu_grad_direct(double x) { return gelu_grad_f64(x); }
 
 template <typename T>
-__global__ void gelu_fwd_direct_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n) {
+__global__ void gelu_fwd_direct_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n,
+                                       const int32_t* __restrict__ n_rows_dev,
+                                       int64_t row_len) {
+  n = live_elems(n, n_rows_dev, row_len);
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
     y[i] = gelu_direct(x[i]);
 }
 template <typename T>
 __global__ void gelu_bwd_direct_kernel(const T* __restrict__ dy, const T* __restrict__ x,
-                                       T* __restrict__ dx, int64_t n) {
+                                       T* __restrict__ dx, int64_t n,
+                                       const int32_t* __restrict__ n_rows_dev,
+                                       int64_t row_len) {
+  n = live_elems(n, n_rows_dev, row_len);
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
     dx[i] = dy[i] * gelu_grad_direct(x[i]);
@@ -216,19 +235,28 @@ inline int direct_blocks(int64_t n) {
 
 using namespace fmoe;
 
-extern "C" int fmoe_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream) {
+// The live-row hint is used when whole rows are 16-byte packs; otherwise every
+// element is processed (dead rows hold finite garbage or zeros, never read).
+static bool rows_are_packs(const int32_t* n_rows_dev, int64_t row_len, int64_t n, int dtype) {
+  return n_rows_dev != nullptr && row_len > 0 && n % row_len == 0 &&
+         (row_len * (int64_t)dtype_size(dtype)) % 16 == 0;
+}
+
+extern "C" int fmoe_gelu_fwd(const void* x, void* y, int64_t n, const int32_t* n_rows_dev,
+                             int64_t row_len, int dtype, void* stream) {
   FMOE_REQUIRE(dtype_size(dtype) != 0, FMOE_ERR_INVALID, "gelu_fwd: unknown dtype %d", dtype);
   FMOE_REQUIRE(n >= 0, FMOE_ERR_INVALID, "gelu_fwd: bad size %lld", (long long)n);
   if (n == 0) return FMOE_OK;
   FMOE_REQUIRE(x && y, FMOE_ERR_INVALID, "gelu_fwd: null pointer");
   hipStream_t s = (hipStream_t)stream;
+  if (!rows_are_packs(n_rows_dev, row_len, n, dtype)) n_rows_dev = nullptr;
   if (dtype == FMOE_F32 || dtype == FMOE_F64) {
     if (dtype == FMOE_F32)
       hipLaunchKernelGGL(gelu_fwd_direct_kernel<float>, dim3(direct_blocks(n)), dim3(256), 0, s,
-                         (const float*)x, (float*)y, n);
+                         (const float*)x, (float*)y, n, n_rows_dev, row_len);
     else
       hipLaunchKernelGGL(gelu_fwd_direct_kernel<double>, dim3(direct_blocks(n)), dim3(256), 0, s,
-                         (const double*)x, (double*)y, n);
+                         (const double*)x, (double*)y, n, n_rows_dev, row_len);
     FMOE_LAUNCH_CHECK("gelu_fwd");
     return FMOE_OK;
   }
@@ -239,7 +267,8 @@ extern "C" int fmoe_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void*
   const int64_t n_packs = aligned16(x) && aligned16(y) ? n / 8 : 0;
   if (n_packs > 0)
     hipLaunchKernelGGL(gelu_fwd_lut_kernel, dim3(lut_blocks(n_packs, cus)), dim3(kActThreads),
-                       kTabFwd * 2, s, (const uint4*)x, (uint4*)y, n_packs, which);
+                       kTabFwd * 2, s, (const uint4*)x, (uint4*)y, n_packs, which, n_rows_dev,
+                       row_len / 8);
   const int64_t done = n_packs * 8, rest = n - done;
   if (rest > 0)
     hipLaunchKernelGGL(gelu_fwd_tab_kernel, dim3((unsigned)((rest + 255) / 256)),
@@ -249,20 +278,23 @@ extern "C" int fmoe_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void*
   return FMOE_OK;
 }
 
-extern "C" int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, int dtype,
+extern "C" int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n,
+                             const int32_t* n_rows_dev, int64_t row_len, int dtype,
                              void* stream) {
   FMOE_REQUIRE(dtype_size(dtype) != 0, FMOE_ERR_INVALID, "gelu_bwd: unknown dtype %d", dtype);
   FMOE_REQUIRE(n >= 0, FMOE_ERR_INVALID, "gelu_bwd: bad size %lld", (long long)n);
   if (n == 0) return FMOE_OK;
   FMOE_REQUIRE(dy && x && dx, FMOE_ERR_INVALID, "gelu_bwd: null pointer");
   hipStream_t s = (hipStream_t)stream;
+  if (!rows_are_packs(n_rows_dev, row_len, n, dtype)) n_rows_dev = nullptr;
   if (dtype == FMOE_F32 || dtype == FMOE_F64) {
     if (dtype == FMOE_F32)
       hipLaunchKernelGGL(gelu_bwd_direct_kernel<float>, dim3(direct_blocks(n)), dim3(256), 0, s,
-                         (const float*)dy, (const float*)x, (float*)dx, n);
+                         (const float*)dy, (const float*)x, (float*)dx, n, n_rows_dev, row_len);
     else
       hipLaunchKernelGGL(gelu_bwd_direct_kernel<double>, dim3(direct_blocks(n)), dim3(256), 0, s,
-                         (const double*)dy, (const double*)x, (double*)dx, n);
+                         (const double*)dy, (const double*)x, (double*)dx, n, n_rows_dev,
+                         row_len);
     FMOE_LAUNCH_CHECK("gelu_bwd");
     return FMOE_OK;
   }
@@ -276,7 +308,7 @@ extern "C" int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n,
     if (n_packs > 0)
       hipLaunchKernelGGL(gelu_bwd_lut_kernel<__hip_bfloat16>, dim3(lut_blocks(n_packs, cus)),
                          dim3(kActThreads), kTabBwd * 4, s, (const uint4*)dy, (const uint4*)x,
-                         (uint4*)dx, n_packs, which);
+                         (uint4*)dx, n_packs, which, n_rows_dev, row_len / 8);
     if (rest > 0)
       hipLaunchKernelGGL(gelu_bwd_tab_kernel<__hip_bfloat16>,
                          dim3((unsigned)((rest + 255) / 256)), dim3(256), 0, s,
@@ -286,7 +318,7 @@ extern "C" int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n,
     if (n_packs > 0)
       hipLaunchKernelGGL(gelu_bwd_lut_kernel<__half>, dim3(lut_blocks(n_packs, cus)),
                          dim3(kActThreads), kTabBwd * 4, s, (const uint4*)dy, (const uint4*)x,
-                         (uint4*)dx, n_packs, which);
+                         (uint4*)dx, n_packs, which, n_rows_dev, row_len / 8);
     if (rest > 0)
       hipLaunchKernelGGL(gelu_bwd_tab_kernel<__half>, dim3((unsigned)((rest + 255) / 256)),
                          dim3(256), 0, s, (const __half*)dy + done, (const uint16_t*)x + done,

@@ -475,20 +475,27 @@ def topk_softmax_bwd(dscore: torch.Tensor, score: torch.Tensor, idx: torch.Tenso
     return dlogits
 
 
-def gelu_fwd(x: torch.Tensor) -> torch.Tensor:
+def _row_len(x: torch.Tensor) -> int:
+    return x.shape[-1] if x.dim() >= 1 and x.numel() else 0
+
+
+def gelu_fwd(x: torch.Tensor, n_rows_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
     """gelu(x) = 0.5 x (1 + erf(x / sqrt 2)), the torch.nn.GELU() between the two
-    expert layers (fmoe/transformer.py:28-30)."""
+    expert layers (fmoe/transformer.py:28-30).  `n_rows_dev` (device int32[1]):
+    only that many leading rows of x are live; the rest of the result is left
+    unwritten."""
     _dev(x, "x")
     _need(x.is_contiguous(), "x must be contiguous")
     y = torch.empty_like(x)
     with _launch(x, "gelu_fwd"):
-        _lib.check(_L.fmoe_gelu_fwd(x.data_ptr(), y.data_ptr(), x.numel(), _dt(x, "x"),
-                                    _stream(x)), "gelu_fwd")
+        _lib.check(_L.fmoe_gelu_fwd(x.data_ptr(), y.data_ptr(), x.numel(), _ptr(n_rows_dev),
+                                    _row_len(x), _dt(x, "x"), _stream(x)), "gelu_fwd")
     return y
 
 
-def gelu_bwd(dy: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
-    """dy * gelu'(x)."""
+def gelu_bwd(dy: torch.Tensor, x: torch.Tensor,
+             n_rows_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dy * gelu'(x); `n_rows_dev` as in gelu_fwd."""
     _dev(x, "x")
     _dev(dy, "dy", x.dtype)
     _need(x.is_contiguous() and dy.is_contiguous() and dy.numel() == x.numel(),
@@ -496,7 +503,8 @@ def gelu_bwd(dy: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     dx = torch.empty_like(x)
     with _launch(x, "gelu_bwd"):
         _lib.check(_L.fmoe_gelu_bwd(dy.data_ptr(), x.data_ptr(), dx.data_ptr(), x.numel(),
-                                    _dt(x, "x"), _stream(x)), "gelu_bwd")
+                                    _ptr(n_rows_dev), _row_len(x), _dt(x, "x"), _stream(x)),
+                   "gelu_bwd")
     return dx
 
 

@@ -217,24 +217,27 @@ class Gelu(Function):
     one kernel each way."""
 
     @staticmethod
-    def forward(ctx, x):
+    def forward(ctx, x, n_rows_dev=None):
         x = x.contiguous()
         ctx.save_for_backward(x)
-        return fmoe_cuda.gelu_fwd(x)
+        ctx.n_rows_dev = n_rows_dev
+        return fmoe_cuda.gelu_fwd(x, n_rows_dev)
 
     @staticmethod
     def backward(ctx, grad_y):
         (x,) = ctx.saved_tensors
-        return fmoe_cuda.gelu_bwd(grad_y.contiguous(), x)
+        return fmoe_cuda.gelu_bwd(grad_y.contiguous(), x, ctx.n_rows_dev), None
 
 
-def apply_activation(activation, x):
+def apply_activation(activation, x, n_rows_dev=None):
     r"""`activation(x)`; an exact torch.nn.GELU on a GPU tensor runs as the
-    library's kernel, anything else as the module itself."""
+    library's kernel, anything else as the module itself.  `n_rows_dev` (device
+    int32[1], optional): the rows of x behind that count are dead (slots a
+    capacity limit dropped) and the kernel skips them."""
     if (type(activation) is torch.nn.GELU and getattr(activation, "approximate", "none") == "none"
             and x.is_cuda and x.dtype in (torch.float32, torch.float64, torch.float16,
                                           torch.bfloat16)):
-        return Gelu.apply(x)
+        return Gelu.apply(x, n_rows_dev)
     return activation(x)
 
 

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .functions import apply_activation
+from .functions import SegmentTable, apply_activation
 from .layers import FMoE
 from .linear import FMoELinear
 
@@ -24,7 +24,9 @@ class _Expert(nn.Module):
 
     def forward(self, inp, fwd_expert_count):
         x = self.htoh4(inp, fwd_expert_count)
-        x = apply_activation(self.activation, x)
+        # with a device-side segment table, the activation skips the dead rows
+        live = fwd_expert_count.seg_off[-1:] if isinstance(fwd_expert_count, SegmentTable) else None
+        x = apply_activation(self.activation, x, live)
         return self.h4toh(x, fwd_expert_count)
 
 

@@ -273,13 +273,17 @@ int fmoe_topk_softmax_bwd(const void* dscore, const void* score, const int64_t* 
  * transformer.py:45 (the reference calls the torch module; these kernels take
  * its place on the GPU).  bf16/f16 read gelu(x) (computed in double precision,
  * rounded once) and gelu'(-|x|) (f32) from tables held in LDS; f32/f64 evaluate
- * erf.  Inputs and outputs must not overlap.  The first 16-bit call on a
- * GPU builds that GPU's tables on `stream`; first calls on one GPU must not come
- * from two streams at once.
+ * erf.  Inputs and outputs must not overlap.  n_rows_dev (DEVICE int32, may be
+ * NULL) with row_len tells that only the first *n_rows_dev rows of row_len
+ * elements are live, as in the expert-ordered buffers behind a capacity limit:
+ * the rest is neither read nor written.  The first 16-bit call on a GPU builds
+ * that GPU's tables on `stream`; first calls on one GPU must not come from two
+ * streams at once.
  */
-int fmoe_gelu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream);
-int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, int dtype,
-                  void* stream);
+int fmoe_gelu_fwd(const void* x, void* y, int64_t n, const int32_t* n_rows_dev,
+                  int64_t row_len, int dtype, void* stream);
+int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n,
+                  const int32_t* n_rows_dev, int64_t row_len, int dtype, void* stream);
 
 /*
  * Selects the grouped-GEMM kernel family: 0 = automatic (MFMA where the shape

@@ -114,3 +114,38 @@ def test_expert_module_uses_the_kernel_only_for_exact_gelu():
     assert seen == ["gelu_fwd", "gelu_bwd"]
     want = O.gelu_backward(np.ones(x.numel()), x.detach().double().cpu().numpy().ravel())
     assert np.abs(x.grad.double().cpu().numpy().ravel() - want).max() <= 2.0 ** -8 * 1.2
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f32"])
+def test_live_row_hint_skips_dead_rows(dt):
+    """With a device-side count of live rows only those rows are computed; the
+    rest of the output is left as it was."""
+    from fastmoe_amd import fmoe_cuda
+    from fastmoe_amd.fmoe_cuda import _L, _dt, _lib, _stream
+
+    dtype = DTYPES[dt]
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(37, 64, generator=g).to(dtype).cuda()
+    dy = torch.randn(37, 64, generator=g).to(dtype).cuda()
+    full_y = fmoe_cuda.gelu_fwd(x)
+    full_dx = fmoe_cuda.gelu_bwd(dy, x)
+    for live in (0, 1, 20, 37, 50):
+        n_rows = torch.tensor([live], dtype=torch.int32, device="cuda")
+        y = torch.full_like(x, 7.0)
+        dx = torch.full_like(x, 7.0)
+        _lib.check(_L.fmoe_gelu_fwd(x.data_ptr(), y.data_ptr(), x.numel(), n_rows.data_ptr(), 64,
+                                    _dt(x, "x"), _stream(x)), "gelu_fwd")
+        _lib.check(_L.fmoe_gelu_bwd(dy.data_ptr(), x.data_ptr(), dx.data_ptr(), x.numel(),
+                                    n_rows.data_ptr(), 64, _dt(x, "x"), _stream(x)), "gelu_bwd")
+        k = min(live, 37)
+        assert torch.equal(y[:k], full_y[:k]) and torch.equal(dx[:k], full_dx[:k])
+        assert (y[k:] == 7.0).all() and (dx[k:] == 7.0).all()
+    # through the binding the hint rides on the autograd function
+    from fastmoe_amd.functions import apply_activation
+    xr = x.clone().requires_grad_(True)
+    n_rows = torch.tensor([20], dtype=torch.int32, device="cuda")
+    out = apply_activation(torch.nn.GELU(), xr, n_rows)
+    out[:20].float().sum().backward()
+    assert torch.equal(out[:20], full_y[:20])
+    ones = torch.ones_like(x)
+    assert torch.equal(xr.grad[:20], fmoe_cuda.gelu_bwd(ones, x)[:20])
