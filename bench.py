@@ -17,7 +17,7 @@ already resident in HBM.  Prints ONE JSON line:
                       pass with events around every op (the dominant op's entry
                       comes from the timed region)
 
-usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2]
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg4]
 """
 from __future__ import annotations
 
@@ -251,7 +251,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", default="cfg2", choices=sorted(CONFIGS))
+    ap.add_argument("--config", default="cfg4", choices=sorted(CONFIGS),
+                    help="workload; the default is the largest single-GPU configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--graph", action="store_true",
                     help="also time the same steps replayed from one HIP graph (extra field)")

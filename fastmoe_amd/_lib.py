@@ -77,12 +77,22 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
     global _lib
     if _lib is not None:
         return _lib
+    from . import build as _build
+
     if not os.path.exists(LIB_PATH):
         if not build_if_missing:
             raise ImportError(f"{LIB_PATH} is missing; run `python fastmoe_amd/build.py`")
-        from . import build as _build
-
         _build.build(verbose=False)
+    elif os.path.isdir(_build.CSRC):
+        # a binary left behind by an earlier state of csrc/ must not be loaded
+        # silently: the kernels and the signature table below would disagree
+        want, have = _build.source_hash(), _build.built_hash(LIB_PATH)
+        if want != have:
+            if not (build_if_missing and os.path.exists(_build.HIPCC)):
+                raise ImportError(
+                    f"{LIB_PATH} was built from other sources (digest {have}, csrc/ has "
+                    f"{want}); run `python fastmoe_amd/build.py`")
+            _build.build(verbose=False)
     _preload_torch_hip_runtime()
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():

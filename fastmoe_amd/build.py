@@ -20,7 +20,9 @@ LIB_PATH = os.path.join(LIB_DIR, "libfmoe_hip.so")
 
 SOURCES = ["api.hip", "route.hip", "dispatch.hip", "gate.hip", "act.hip", "gemm_simt.hip", "gemm_mfma.hip",
            "gemm_mfma_wide.hip"]
-HEADERS = ["common.h", "gemm.h", os.path.join("..", "..", "include", "fmoe_hip.h")]
+HEADERS = ["common.h", "gemm.h", "dma_desc.h", os.path.join("..", "..", "include", "fmoe_hip.h")]
+# the library carries a digest of the files it was built from behind this marker
+HASH_MARKER = "fmoe-src:"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -36,9 +38,33 @@ FLAGS = [
 ]
 
 
+def source_hash() -> str:
+    """Digest (12 hex digits) of every source and header the library is built from."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in SOURCES + HEADERS:
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read() + b"\0")
+    return h.hexdigest()[:12]
+
+
+def built_hash(lib_path: str = LIB_PATH):
+    """The digest a built library carries, read from the file without loading it
+    (None if the file has none)."""
+    with open(lib_path, "rb") as f:
+        blob = f.read()
+    at = blob.find(HASH_MARKER.encode())
+    if at < 0:
+        return None
+    return blob[at + len(HASH_MARKER):at + len(HASH_MARKER) + 12].decode("ascii", "replace")
+
+
 def _compile(src: str, verbose: bool) -> str:
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
     cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    if src == "api.hip":
+        cmd.insert(-4, f'-DFMOE_SOURCE_HASH="{source_hash()}"')
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -12,6 +12,8 @@
 // 0.5 x (1 + erf(x / sqrt 2)) directly.
 #include <math.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace fmoe {
@@ -186,21 +188,31 @@ __global__ void gelu_bwd_direct_kernel(const T* __restrict__ dy, const T* __rest
 
 // ---- host side ------------------------------------------------------------
 constexpr int kMaxDevices = 64;
+std::mutex g_setup_mutex;          // guards everything below
 bool g_tables_built[kMaxDevices];
 bool g_lds_configured = false;
 int g_cu_count[kMaxDevices];
 
-// Builds the tables of the current device on `s` the first time it is seen.
-// The first calls on a device must not come from two streams at once.
+// Builds the tables of the current device the first time a 16-bit call reaches
+// it, on `s`, and waits for them: from then on any stream may read them.  A
+// first call under stream capture is refused (the tables would exist only once
+// the graph has been replayed): run one eager call before capturing.
 int ensure_tables(hipStream_t s, int* cu_count) {
   int dev = 0;
   FMOE_HIP_CHECK(hipGetDevice(&dev));
   FMOE_REQUIRE(dev >= 0 && dev < kMaxDevices, FMOE_ERR_UNSUPPORTED, "gelu: device %d", dev);
+  std::lock_guard<std::mutex> lock(g_setup_mutex);
   if (!g_tables_built[dev]) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    FMOE_HIP_CHECK(hipStreamIsCapturing(s, &capture));
+    FMOE_REQUIRE(capture == hipStreamCaptureStatusNone, FMOE_ERR_UNSUPPORTED,
+                 "gelu: the first 16-bit call on a device builds its tables and cannot be "
+                 "captured into a graph; make one eager call first");
     FMOE_HIP_CHECK(hipDeviceGetAttribute(&g_cu_count[dev], hipDeviceAttributeMultiprocessorCount,
                                          dev));
     hipLaunchKernelGGL(gelu_table_kernel, dim3(kTabFwd / 256), dim3(256), 0, s);
     FMOE_LAUNCH_CHECK("gelu_table");
+    FMOE_HIP_CHECK(hipStreamSynchronize(s));
     g_tables_built[dev] = true;
   }
   if (!g_lds_configured) {

@@ -125,7 +125,14 @@ static int run_gemm(int mode, const GemmArgs& g, int dtype, hipStream_t s) {
 
 using namespace fmoe;
 
-extern "C" const char* fmoe_version(void) { return "fastmoe_amd 0.1 (gfx950)"; }
+#ifndef FMOE_SOURCE_HASH
+#define FMOE_SOURCE_HASH "unknown"
+#endif
+// the build script puts a digest of the sources behind the "fmoe-src:" marker, so
+// that a loader can tell a library built from other sources without loading it
+extern "C" const char* fmoe_version(void) {
+  return "fastmoe_amd 0.2 (gfx950) fmoe-src:" FMOE_SOURCE_HASH;
+}
 extern "C" const char* fmoe_last_error(void) { return g_err; }
 
 extern "C" int fmoe_set_gemm_path(int path) {

@@ -6,6 +6,8 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../include/fmoe_hip.h"
 
 namespace fmoe {
@@ -37,6 +39,20 @@ inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
     if (_e != hipSuccess)                                                  \
       return ::fmoe::set_error(FMOE_ERR_HIP, "launch of %s failed: %s", name, \
                                hipGetErrorString(_e));                     \
+  } while (0)
+
+// Raises a kernel's dynamic-LDS limit once per process (the attribute belongs to
+// the function); safe when several host threads make their first call at once.
+#define FMOE_SET_DYNAMIC_LDS_ONCE(kern, bytes)                                          \
+  do {                                                                                  \
+    static std::once_flag _once;                                                        \
+    static hipError_t _once_err = hipSuccess;                                           \
+    std::call_once(_once, [&] {                                                         \
+      _once_err = hipFuncSetAttribute((const void*)(kern),                              \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize,       \
+                                      (int)(bytes));                                    \
+    });                                                                                 \
+    FMOE_HIP_CHECK(_once_err);                                                          \
   } while (0)
 
 inline size_t dtype_size(int dtype) {

@@ -20,8 +20,13 @@ constexpr int kGateThreads = 256;
 constexpr int kGateWideFrom = 64;
 constexpr int kGateChunk = 8;                       // logits a lane loads before it sorts them
 
+// Order of the candidates: larger logit first, equal logits by expert index.
+// A NaN logit ranks above every number (as torch.topk ranks it), so a diverged
+// row selects its NaNs and its scores come out as NaN instead of being masked.
 template <typename A>
 __device__ __forceinline__ bool better(A v, int e, A w, int f) {
+  const bool v_nan = v != v, w_nan = w != w;
+  if (v_nan || w_nan) return v_nan && (!w_nan || e < f);
   return v > w || (v == w && e < f);
 }
 

@@ -38,6 +38,7 @@
 // reference; the per-expert cuBLAS loop there becomes a tile index space.
 #include <type_traits>
 
+#include "dma_desc.h"
 #include "gemm.h"
 
 namespace fmoe {
@@ -63,7 +64,7 @@ template <> struct Mma<__half> {
   }
 };
 
-constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any num_records used here
+constexpr uint32_t kOutOfRange = kDmaOutOfRange;  // beyond any num_records used here
 constexpr int kRsrcFlags = 0x00020000;         // raw buffer, 32-bit data format
 
 // One operand tile of R rows (the M or N index) by BK values of K.
@@ -99,7 +100,7 @@ struct DmaTile {
   uint32_t voff[kPerWave];
   // per wave (scalar registers)
   i32x4_t rsrc;       // buffer descriptor of the current slice; num_records ends the valid data
-  int remaining;      // bytes from the slice origin to the end of the valid data
+  int64_t remaining;  // bytes from the slice origin to the end of the valid data (can pass 2^31)
   int step;           // bytes between consecutive slices
   int k_left;         // K values from the slice start to the end of K
 
@@ -121,16 +122,15 @@ struct DmaTile {
       }
     }
     // everything past the ragged edge is beyond num_records and reads as zero
-    remaining = KC ? ((r_valid - 1) * ld + k_total) * 2
-                   : ((k_total - 1) * ld + r_span) * 2;
-    if (k_total <= 0) remaining = 0;
-    remaining = __builtin_amdgcn_readfirstlane(remaining);
+    const int64_t bytes = dma_valid_bytes(KC, r_valid, r_span, ld, k_total);
+    remaining = ((int64_t)__builtin_amdgcn_readfirstlane((int)(bytes >> 32)) << 32) |
+                (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)bytes);
     step = __builtin_amdgcn_readfirstlane((KC ? BK : BK * ld) * 2);
     k_left = k_total;
     const uint64_t p = (uint64_t)origin;
     rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
     rsrc[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32) & 0xffff);  // stride 0
-    rsrc[2] = max(remaining, 0);
+    rsrc[2] = dma_num_records(remaining);
     rsrc[3] = kRsrcFlags;
     mask_k_tail(wave, lane);
   }
@@ -153,7 +153,7 @@ struct DmaTile {
     rsrc[0] = (int)(uint32_t)p;
     rsrc[1] = (int)(uint32_t)(p >> 32);
     remaining -= step;
-    rsrc[2] = max(remaining, 0);
+    rsrc[2] = dma_num_records(remaining);
     k_left -= BK;
     mask_k_tail(wave, lane);
   }
@@ -879,13 +879,7 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
   auto kern = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, NS, MODE>;
-  static bool configured = false;  // attribute is per function, set once
-  if (!configured) {
-    FMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes));
-    configured = true;
-  }
+  FMOE_SET_DYNAMIC_LDS_ONCE(kern, lds_bytes);
   int tiles_n, tiles_m;
   int64_t blocks;
   if (MODE == GEMM_WGRAD) {
@@ -970,13 +964,7 @@ static int launch_bwd_fused(const GemmArgs& gd, const GemmArgs& gw, hipStream_t 
   constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
   auto kern = gemm_bwd_kernel<T, BM, BN, BK, WM, WN, NS>;
-  static bool configured = false;  // attribute is per function, set once
-  if (!configured) {
-    FMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes));
-    configured = true;
-  }
+  FMOE_SET_DYNAMIC_LDS_ONCE(kern, lds_bytes);
   const int tiles_n_d = ceil_div(gd.in_feat, BN);
   const int tiles_n_w = ceil_div(gw.in_feat, BN), tiles_m_w = ceil_div(gw.out_feat, BM);
   int64_t blocks = (int64_t)tiles_n_d * (gd.n_rows / BM + (int64_t)gd.n_expert) +
@@ -1016,8 +1004,7 @@ bool gemm_mfma_supported(int mode, const GemmArgs& g, int dtype) {
   if (dtype != FMOE_BF16 && dtype != FMOE_F16) return false;
   if (g.in_feat % 8 != 0 || g.out_feat % 8 != 0) return false;
   // tile-relative byte offsets are 32-bit: 256 rows of either feature size
-  if ((int64_t)g.in_feat * 512 >= (int64_t)kOutOfRange ||
-      (int64_t)g.out_feat * 512 >= (int64_t)kOutOfRange) return false;
+  if (!dma_ld_supported(g.in_feat) || !dma_ld_supported(g.out_feat)) return false;
   if (((uintptr_t)g.a | (uintptr_t)g.b | (uintptr_t)g.c) % 16 != 0) return false;
   return true;
 }

@@ -292,12 +292,7 @@ int launch_wide_mode(const GemmArgs& g, hipStream_t s) {
   constexpr size_t lds = wide_lds_bytes<F>();
   static_assert(2 * lds <= 160 * 1024, "at least two blocks per gfx950 CU");
   auto kern = gemm_wide_kernel<F, MODE>;
-  static bool configured = false;  // attribute is per function, set once
-  if (!configured) {
-    FMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    configured = true;
-  }
+  FMOE_SET_DYNAMIC_LDS_ONCE(kern, lds);
   dim3 grid;
   if (MODE == GEMM_WGRAD) {
     grid = dim3(ceil_div(g.in_feat, kWideTile), ceil_div(g.out_feat, kWideTile), g.n_expert);

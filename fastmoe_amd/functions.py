@@ -130,9 +130,9 @@ class RoutePlan:
     """Everything the dispatch needs about one routing decision."""
 
     def __init__(self, gate: torch.Tensor, num_expert: int):
-        self.top_k = gate.shape[1] if gate.dim() == 2 else 1
-        self.n_tokens = gate.shape[0]
+        self.top_k = gate.shape[-1] if gate.dim() >= 2 else 1
         self.n_slots = gate.numel()
+        self.n_tokens = self.n_slots // max(self.top_k, 1)
         with torch.no_grad():
             pos, counts, seg_off, inv = fmoe_cuda.route(gate.contiguous(), num_expert)
         self.pos = pos
@@ -243,8 +243,10 @@ def apply_activation(activation, x, n_rows_dev=None):
 
 def topk_softmax(logits, top_k: int):
     r"""Top-k gate decision of logits [..., E]: `(idx [T, k] int64, score [T, k])`.
-    On the GPU (and for k up to fmoe_cuda.MAX_GATE_TOP_K) one fused kernel; anywhere
-    else the torch.topk + softmax formulation of the reference."""
+    On the GPU, for k up to fmoe_cuda.MAX_GATE_TOP_K, one fused kernel each way.
+    The gate is host-side torch code in the reference (naive_gate.py:31-38), and a
+    gate module may live on the CPU or ask for a larger k: those two cases keep the
+    reference's own torch.topk + softmax formulation."""
     flat = logits.reshape(-1, logits.shape[-1])
     if flat.is_cuda and top_k <= fmoe_cuda.MAX_GATE_TOP_K and flat.dtype in (
             torch.float32, torch.float64, torch.float16, torch.bfloat16):

@@ -124,7 +124,9 @@ class FMoE(nn.Module):
         mark_module_parallel_comm(self.gate, "gate")
 
     def _device_side_dispatch(self) -> bool:
-        return self.experts_fused and getattr(self.experts, "accepts_segment_table", False)
+        # the fused combine kernels keep a token's slots in the lanes of one wave
+        return (self.experts_fused and self.top_k <= 64
+                and getattr(self.experts, "accepts_segment_table", False))
 
     # ------------------------------------------------------------- forward
     def forward(self, moe_inp):

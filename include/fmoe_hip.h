@@ -249,7 +249,8 @@ int fmoe_seg_off_from_host_counts(const int64_t* expert_count_host,
  *   score[t][j] = exp(v_j - v_0) / sum_i exp(v_i - v_0)      (dtype of the logits)
  * Replaces torch.topk + F.softmax of fmoe/gates/naive_gate.py:31-38; torch.topk
  * leaves the order of its results open, this call returns them by descending
- * logit.  top_k <= min(n_expert, FMOE_MAX_GATE_TOP_K); NaN logits are never picked.
+ * logit.  top_k <= min(n_expert, FMOE_MAX_GATE_TOP_K).  A NaN logit ranks above
+ * every number, as in torch.topk, so a token with NaN logits gets NaN scores.
  */
 int fmoe_topk_softmax_fwd(const void* logits, int64_t n_tokens, int32_t n_expert,
                           int32_t top_k, int64_t* idx, void* score, int dtype,
@@ -277,8 +278,8 @@ int fmoe_topk_softmax_bwd(const void* dscore, const void* score, const int64_t* 
  * NULL) with row_len tells that only the first *n_rows_dev rows of row_len
  * elements are live, as in the expert-ordered buffers behind a capacity limit:
  * the rest is neither read nor written.  The first 16-bit call on a GPU builds
- * that GPU's tables on `stream`; first calls on one GPU must not come from two
- * streams at once.
+ * that GPU's tables on `stream` and waits for them (thread-safe); that one call
+ * cannot be captured into a HIP graph and returns FMOE_ERR_UNSUPPORTED there.
  */
 int fmoe_gelu_fwd(const void* x, void* y, int64_t n, const int32_t* n_rows_dev,
                   int64_t row_len, int dtype, void* stream);

@@ -86,6 +86,34 @@ def test_ties_and_minus_infinity_in_a_wide_expert_set():
     assert np.abs(score.double().cpu().numpy() - want).max() <= 1e-6
 
 
+def test_nan_logits_rank_first_as_in_torch_topk():
+    """torch.topk ranks NaN above every number (naive_gate.py:31-38 inherits that):
+    a NaN logit is selected and the token's scores become NaN, for both the
+    register-resident (<= 512 experts) and the sorted-list kernels."""
+    from fastmoe_amd import fmoe_cuda
+
+    nan, ninf = float("nan"), float("-inf")
+    for e in (6, 600):
+        lt = torch.zeros(4, e)
+        lt[0, :6] = torch.tensor([1.0, nan, 3.0, ninf, 2.0, 0.5])
+        lt[1, :6] = torch.tensor([nan, nan, nan, 1.0, ninf, 0.0])     # fewer numbers than k
+        lt[2, :6] = torch.tensor([ninf, ninf, 1.0, ninf, ninf, ninf])
+        lt[3, :6] = torch.tensor([5.0, 4.0, 3.0, 2.0, 1.0, 0.5])
+        lt[:, 6:] = -10.0
+        idx, score = fmoe_cuda.topk_softmax_fwd(lt.cuda(), 3)
+        tval, tidx = torch.topk(lt, 3, dim=-1)
+        idx, score = idx.cpu(), score.cpu()
+        assert idx[0].tolist() == [1, 2, 4] and idx[1].tolist() == [0, 1, 2]
+        assert idx[2, 0].item() == 2 and idx[3].tolist() == [0, 1, 2]
+        for r in range(4):                      # same experts as torch.topk picks
+            assert sorted(idx[r].tolist()) == sorted(tidx[r].tolist()) or r == 2
+        assert idx.min().item() >= 0 and idx.max().item() < e
+        assert torch.isnan(score[0]).all() and torch.isnan(score[1]).all()
+        want = F.softmax(tval[3].double(), dim=-1)
+        assert (score[3].double() - want).abs().max().item() <= 1e-6
+        assert not torch.isnan(score[2:]).any()
+
+
 def test_autograd_matches_torch_formulation():
     """The fused op inside autograd against torch.topk + softmax (no ties)."""
     from fastmoe_amd.functions import topk_softmax

@@ -117,3 +117,79 @@ def test_bench_workloads_are_seeded_and_shaped():
     work = bench.kernel_work(bench.CONFIGS["cfg2"], 16384)
     assert work["grouped_linear_fwd"] == ("flop", 2.0 * 16384 * 1024 * 4096)
     assert work["local_scatter"][1] == 2.0 * 16384 * 1024 * 2 + 8.0 * 16384
+
+
+def _descriptor_checker(tmp_path):
+    """Compiles the grouped GEMM's descriptor arithmetic (csrc/dma_desc.h) for the
+    host and hands back its three functions."""
+    import ctypes
+    import os
+    import subprocess
+
+    from conftest import ROOT
+
+    src = tmp_path / "dma_desc_host.cpp"
+    src.write_text(
+        '#include "dma_desc.h"\n'
+        'extern "C" long long valid_bytes(int kc, int rv, int rs, int ld, int kt) {\n'
+        '  return fmoe::dma_valid_bytes(kc != 0, rv, rs, ld, kt); }\n'
+        'extern "C" int num_records(long long r) { return fmoe::dma_num_records(r); }\n'
+        'extern "C" int ld_ok(long long ld) { return fmoe::dma_ld_supported(ld); }\n')
+    so = tmp_path / "dma_desc_host.so"
+    subprocess.run(["g++", "-O1", "-shared", "-fPIC", "-I",
+                    os.path.join(ROOT, "fastmoe_amd", "csrc"), str(src), "-o", str(so)], check=True)
+    lib = ctypes.CDLL(str(so))
+    lib.valid_bytes.restype = ctypes.c_longlong
+    lib.valid_bytes.argtypes = [ctypes.c_int] * 5
+    lib.num_records.argtypes = [ctypes.c_longlong]
+    lib.ld_ok.argtypes = [ctypes.c_longlong]
+    return lib
+
+
+def test_gemm_descriptors_survive_experts_beyond_2_to_the_31_bytes(tmp_path):
+    """The weight-gradient product walks the rows of one expert as its K index:
+    rows x features x 2 bytes passes 2^31 for a long expert.  The byte count must
+    stay exact (64-bit) and the descriptor's 32-bit num_records must neither wrap
+    nor cut off rows that exist; rows past the end must still read as zeros."""
+    lib = _descriptor_checker(tmp_path)
+    out_of_range = 0x80000000
+    for rows, ld, bk in ((300000, 4096, 32), (75000, 14336, 64), (1 << 20, 16384, 64),
+                         (1000, 1024, 32)):
+        r_span = min(256, ld)
+        total = lib.valid_bytes(0, r_span, r_span, ld, rows)
+        assert total == ((rows - 1) * ld + r_span) * 2          # exact, no wrap
+        step = bk * ld * 2
+        for t in (0, 1, (rows // bk) // 2, rows // bk - 1, rows // bk, rows // bk + 1):
+            remaining = total - t * step
+            rec = lib.num_records(remaining)
+            assert 0 <= rec < out_of_range
+            k_left = rows - t * bk
+            for k in range(bk):
+                first = (k * ld) * 2                             # first pack of K row k
+                last = (k * ld + r_span - 8) * 2                 # last valid pack of it
+                assert last + 16 < out_of_range
+                if k < k_left:
+                    assert last + 16 <= rec, (rows, ld, t, k)    # existing rows are readable
+                else:
+                    assert first >= rec, (rows, ld, t, k)        # rows past the end are not
+    # [row][k] operands: 256 rows of the widest supported feature size
+    ld = (out_of_range // 512) - 8
+    assert lib.ld_ok(ld) and not lib.ld_ok(out_of_range // 512)
+    total = lib.valid_bytes(1, 256, 0, ld, ld)
+    assert total == (255 * ld + ld) * 2 and lib.num_records(total) == total
+    assert lib.num_records(0) == 0 and lib.num_records(-4096) == 0
+    assert lib.valid_bytes(0, 256, 256, 4096, 0) == 0            # expert without rows
+
+
+def test_stale_library_is_detected(tmp_path):
+    """A binary built from other sources is told apart without loading it."""
+    from fastmoe_amd import _lib, build
+
+    assert build.built_hash(_lib.LIB_PATH) == build.source_hash()
+    assert build.source_hash().encode() in _lib.load().fmoe_version()
+    fake = tmp_path / "libfmoe_hip.so"
+    blob = open(_lib.LIB_PATH, "rb").read()
+    marker = build.HASH_MARKER.encode()
+    at = blob.find(marker) + len(marker)
+    fake.write_bytes(blob[:at] + b"0" * 12 + blob[at + 12:])
+    assert build.built_hash(str(fake)) == "0" * 12 != build.source_hash()
