@@ -24,6 +24,8 @@ SIGNATURES = {
                                 c_void_p, c_int64, c_void_p]),
     "fmoe_route": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p,
                            c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
+    "fmoe_route_static": (c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_void_p]),
     "fmoe_limit_by_capacity": (c_int, [c_void_p, c_void_p, c_void_p, c_int64,
                                        c_int64, c_void_p]),
     "fmoe_prune_gate_by_capacity": (c_int, [c_void_p, c_void_p, c_void_p, c_int64,

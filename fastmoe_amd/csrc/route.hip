@@ -224,6 +224,33 @@ __global__ __launch_bounds__(256) void limit_by_capacity_kernel(
 }
 
 // --------------------------------------------------------------- host side
+// Scratch of the entry point that allocates nothing (fmoe_route_static): the
+// per-block histograms live in this array instead of a caller's workspace.
+// Every GPU the library runs on holds its own copy until the process ends.
+constexpr int64_t kStaticScratchBytes = FMOE_ROUTE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxRouteDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxRouteDevices];   // device address of `scratch`, per GPU
+
+// Device address of the current GPU's copy of `scratch` (looked up once per GPU).
+static int static_scratch(void** out) {
+  int dev = 0;
+  FMOE_HIP_CHECK(hipGetDevice(&dev));
+  FMOE_REQUIRE(dev >= 0 && dev < kMaxRouteDevices, FMOE_ERR_UNSUPPORTED,
+               "route_static: device %d", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    FMOE_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    FMOE_REQUIRE(p != nullptr, FMOE_ERR_HIP, "route_static: scratch has no device address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return FMOE_OK;
+}
+
 struct RouteWs {
   int32_t* block_hist;
   int32_t* cap_copy;
@@ -326,6 +353,25 @@ extern "C" int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
     FMOE_LAUNCH_CHECK("route_place");
   }
   return FMOE_OK;
+}
+
+extern "C" int fmoe_route_static(const int64_t* gate, int64_t numel, int32_t n_expert,
+                                 int64_t* count64, int32_t* seg_off, int64_t* pos,
+                                 int32_t* inv, void* stream) {
+  int rc = check_route_args(numel, n_expert);
+  if (rc) return rc;
+  const int64_t need = route_ws_bytes(numel, n_expert);
+  FMOE_REQUIRE(need <= kStaticScratchBytes, FMOE_ERR_WORKSPACE,
+               "route_static: %lld slots x %d experts need %lld bytes of scratch, the "
+               "built-in buffer holds %lld; use fmoe_route with a workspace",
+               (long long)numel, n_expert, (long long)need, (long long)kStaticScratchBytes);
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc) return rc;
+  // every block of the histogram kernel overwrites its whole row of the table
+  // before anything reads it, so what the last call left behind needs no clearing
+  return fmoe_route(gate, numel, n_expert, count64, seg_off, pos, inv, ws, kStaticScratchBytes,
+                    stream);
 }
 
 extern "C" int fmoe_assign_pos(int32_t* cum_count, const int64_t* gate,

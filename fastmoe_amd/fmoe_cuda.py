@@ -316,6 +316,29 @@ def route(gate: torch.Tensor, n_expert: int, want_inv: bool = True
     return pos, count, seg, inv
 
 
+def route_static(gate: torch.Tensor, n_expert: int, count: torch.Tensor, seg_off: torch.Tensor,
+                 pos: torch.Tensor, inv: Optional[torch.Tensor] = None) -> None:
+    """`route` into tensors the caller already holds, with the library's built-in
+    scratch buffer instead of a workspace: the call itself allocates nothing
+    (fmoe_route_static).  count int64[E], seg_off int32[E+1], pos int64[N],
+    inv int32[N] or None.  Calls on one GPU share the buffer and must not overlap."""
+    _dev(gate, "gate", torch.int64)
+    _dev(count, "count", torch.int64)
+    _dev(seg_off, "seg_off", torch.int32)
+    _dev(pos, "pos", torch.int64)
+    n = gate.numel()
+    _need(count.numel() == n_expert and seg_off.numel() == n_expert + 1 and pos.numel() >= n,
+          "route_static: count[E], seg_off[E+1] and pos[N] expected")
+    if inv is not None:
+        _dev(inv, "inv", torch.int32)
+        _need(inv.numel() >= n, "route_static: inv must have N entries")
+    with _launch(gate, "route"):
+        _lib.check(
+            _L.fmoe_route_static(gate.data_ptr(), n, n_expert, count.data_ptr(),
+                                 seg_off.data_ptr(), pos.data_ptr(), _ptr(inv), _stream(gate)),
+            "route_static")
+
+
 def grouped_linear_fwd(x: torch.Tensor, seg_off: torch.Tensor, weight: torch.Tensor,
                        bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y[seg_e] = x[seg_e] @ weight[e].T + bias[e] with device-side seg_off."""

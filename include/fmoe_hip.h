@@ -103,6 +103,22 @@ int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
                int64_t* count64, int32_t* seg_off, int64_t* pos, int32_t* inv,
                void* workspace, int64_t workspace_bytes, void* stream);
 
+/*
+ * fmoe_route for callers that cannot allocate: the same kernels and results,
+ * with the per-block histograms in a buffer built into the library
+ * (FMOE_ROUTE_STATIC_SCRATCH_BYTES per GPU, held until the process ends) instead
+ * of a workspace argument.  It calls no allocating routine, so it may be used
+ * under HIP graph capture, in serving loops and in harnesses that forbid
+ * hipMalloc.  Sizes whose workspace (fmoe_route_workspace_bytes) exceeds the
+ * buffer are rejected with FMOE_ERR_WORKSPACE.  All calls on one GPU share the
+ * buffer: calls that overlap in time on one GPU (two streams) race.
+ * No counterpart in the reference; it exists for the callers named above.
+ */
+#define FMOE_ROUTE_STATIC_SCRATCH_BYTES (4 * 1024 * 1024)
+int fmoe_route_static(const int64_t* gate, int64_t numel, int32_t n_expert,
+                      int64_t* count64, int32_t* seg_off, int64_t* pos, int32_t* inv,
+                      void* stream);
+
 /* ----------------------------------------------------------------- capacity */
 
 /*
