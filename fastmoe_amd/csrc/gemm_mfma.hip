@@ -4,8 +4,10 @@
 // synchronisation is needed.
 //
 // Block tile BM x BN x BK with WM x WN wave64s; every wave owns a
-// (BM/WM) x (BN/WN) patch as a grid of 32x32 accumulators fed by
-// v_mfma_f32_32x32x16_{bf16,f16}.
+// (BM/WM) x (BN/WN) patch as a grid of 16x16 accumulators fed by
+// v_mfma_f32_16x16x32_{bf16,f16}: on random data the chip is power-limited, and
+// this shape sustains about 16% more FLOP/s than 32x32x16 at the same power
+// (2.07 vs 1.78 PFLOP/s for a loop of MFMAs alone).
 //
 // Operand tiles go from HBM/L2 straight into LDS with buffer_load_dwordx4 ...
 // lds (no staging registers): one wave instruction fills 1 KiB of LDS, lane l
@@ -37,6 +39,7 @@
 // Operand roles follow cuda/parallel_linear.cuh:69-87,124-147 of the
 // reference; the per-expert cuBLAS loop there becomes a tile index space.
 #include <type_traits>
+#include <utility>
 
 #include "dma_desc.h"
 #include "gemm.h"
@@ -45,21 +48,50 @@ namespace fmoe {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
-typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 typedef __attribute__((ext_vector_type(4))) int i32x4_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-template <typename T> struct Mma;
-template <> struct Mma<__hip_bfloat16> {
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop
+// whose counter is a compile-time constant inside the body.
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+// 32x32x16: for the products whose operands need the transposing LDS read (two
+// instructions per fragment); there the 16-cycle MFMAs leave too few issue
+// slots between them, and the 32-cycle shape is the faster one.
+template <typename T> struct Mma32;
+template <> struct Mma32<__hip_bfloat16> {
   __device__ static __forceinline__ f32x16_t run(uint4 a, uint4 b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
         __builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
   }
 };
-template <> struct Mma<__half> {
+template <> struct Mma32<__half> {
   __device__ static __forceinline__ f32x16_t run(uint4 a, uint4 b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(
+        __builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+};
+
+template <typename T> struct Mma;
+template <> struct Mma<__hip_bfloat16> {
+  __device__ static __forceinline__ f32x4_t run(uint4 a, uint4 b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+        __builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<__half> {
+  __device__ static __forceinline__ f32x4_t run(uint4 a, uint4 b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(
         __builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
   }
 };
@@ -117,7 +149,8 @@ struct DmaTile {
         voff[i] = (uint32_t)(row * ld + pack_k(b, lane)) * 2u;
       } else {
         const int k = b * (64 / kRowPacks) + lane / kRowPacks;
-        const int rc = (lane % kRowPacks) ^ ((k & 3) << 2);  // 32-byte segment ^ 2 (k & 3)
+        // 32-byte segment ^ (2 (k & 3) + bit 3 of k), in 16-byte packs
+        const int rc = (lane % kRowPacks) ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1);
         voff[i] = rc * 8 < r_valid ? (uint32_t)(k * ld + rc * 8) * 2u : kOutOfRange;
       }
     }
@@ -172,9 +205,39 @@ struct DmaTile {
                  :: "s"(dst), "v"(voff[i]), "s"(rsrc) : "memory", "m0");
   }
 
+  // MFMA fragment of the 16-row sub-tile starting at `row16`, K step `ks`
+  // (32 values of K): lane l holds row row16 + l%16, K values 8*(l/16) .. +7.
+  __device__ static __forceinline__ uint4 frag(const uint16_t* lds, int row16,
+                                               int ks, int lane) {
+    if (KC) {
+      const int r = row16 + (lane & 15);
+      const int pack = (ks * 4 + (lane >> 4)) ^ row_swizzle(r);
+      return *reinterpret_cast<const uint4*>(lds + r * BK + pack * 8);
+    } else {
+      // ds_read_b64_tr_b16: within 16 lanes, lane i supplies the address of
+      // elements [k + i/4][m + 4*(i%4) .. +3] and receives [k .. k+3][m + i].
+      const int k = ks * 32 + 8 * (lane >> 4) + ((lane & 15) >> 2);
+      const int m = row16 + 4 * (lane & 3);
+      // 32-byte segments; a 64-bit read is served 32 lanes at a time, i.e. two
+      // groups of 16 lanes whose k differ by 8, 4 k-rows each, all in one
+      // segment: XOR with 2 (k & 3) + bit 3 of k puts those 8 chunks into 8
+      // different segments of a 256-byte bank row
+      const int seg = (m >> 4) ^ ((k & 3) << 1) ^ ((k >> 3) & 1), within = m & 15;
+      const uint16_t* p = lds + k * R + seg * 16 + within;
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4_t*)(p));
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4_t*)(p + 4 * R));
+      uint4 out;
+      const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+      out.x = l2.x; out.y = l2.y; out.z = h2.x; out.w = h2.y;
+      return out;
+    }
+  }
+
   // MFMA fragment of the 32-row sub-tile starting at `row32`, K step `kk`
   // (16 values of K): lane l holds row row32 + l%32, K values 8*(l/32) .. +7.
-  __device__ static __forceinline__ uint4 frag(const uint16_t* lds, int row32,
+  __device__ static __forceinline__ uint4 frag32(const uint16_t* lds, int row32,
                                                int kk, int lane) {
     if (KC) {
       const int r = row32 + (lane & 31);
@@ -187,8 +250,8 @@ struct DmaTile {
       const int m = row32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
       // 32-byte segments; a 64-bit read is served 32 lanes at a time, i.e. 4 k-rows
       // x 2 segments: XOR with 2 (k & 3) puts those 8 chunks into 8 different
-      // segments of a 256-byte bank row
-      const int seg = (m >> 4) ^ ((k & 3) << 1), within = m & 15;
+      // segments of a 256-byte bank row (bit 3 of k, constant here, serves frag())
+      const int seg = (m >> 4) ^ ((k & 3) << 1) ^ ((k >> 3) & 1), within = m & 15;
       const uint16_t* p = lds + k * R + seg * 16 + within;
       const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
           (__attribute__((address_space(3))) s16x4_t*)(p));
@@ -236,7 +299,356 @@ struct TileRows {
 // out_feat x in_feat gradient) by columns [n_origin, + BN); `where` names
 // the expert, m0 and the expert's rows.
 template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
-__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
+__device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, TileRows where,
+                                          int n_origin) {
+  constexpr int NW = WM * WN;
+  constexpr int NT = NW * 64;
+  constexpr bool A_KC = MODE != GEMM_WGRAD;
+  constexpr bool B_KC = MODE == GEMM_FWD;
+  constexpr int TM = BM / WM / 16, TN = BN / WN / 16;   // 16x16 blocks of a wave
+  static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0 && BK % 32 == 0, "tile shape");
+  static_assert((NS >= 4 && NS <= 6) || (NS == 2 && BK == 64), "LDS stages");
+  using ATile = DmaTile<BM, BK, NW, A_KC>;
+  using BTile = DmaTile<BN, BK, NW, B_KC>;
+  constexpr int kStageBytes = ATile::kBytes + BTile::kBytes;
+  constexpr int kStageElems = kStageBytes / 2;
+  constexpr int kLoads = ATile::kPerWave + BTile::kPerWave;  // per wave per slice
+  static_assert(NS == 2 || kLoads * (NS - 3) < 64, "vmcnt is a 6-bit counter");
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave / WN, wave_n = wave % WN;
+  const int in_f = g.in_feat, out_f = g.out_feat;
+  const int e = __builtin_amdgcn_readfirstlane(where.e);
+  const int row0 = __builtin_amdgcn_readfirstlane(where.row0);
+  const int cnt = __builtin_amdgcn_readfirstlane(where.cnt);
+
+  int M, N, K, lda, ldb, ldc;
+  const uint16_t *A, *B;
+  T* C;
+  if (MODE == GEMM_FWD) {
+    M = cnt; N = out_f; K = in_f;
+    A = (const uint16_t*)g.a + (int64_t)row0 * in_f;        lda = in_f;
+    B = (const uint16_t*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
+    C = (T*)g.c + (int64_t)row0 * out_f;                    ldc = out_f;
+  } else if (MODE == GEMM_DGRAD) {
+    M = cnt; N = in_f; K = out_f;
+    A = (const uint16_t*)g.a + (int64_t)row0 * out_f;       lda = out_f;
+    B = (const uint16_t*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
+    C = (T*)g.c + (int64_t)row0 * in_f;                     ldc = in_f;
+  } else {
+    M = out_f; N = in_f; K = cnt;
+    A = (const uint16_t*)g.a + (int64_t)row0 * out_f;       lda = out_f;
+    B = (const uint16_t*)g.b + (int64_t)row0 * in_f;        ldb = in_f;
+    C = (T*)g.c + (int64_t)e * out_f * in_f;                ldc = in_f;
+  }
+  const int m0 = __builtin_amdgcn_readfirstlane(where.m0);
+  const int n0 = __builtin_amdgcn_readfirstlane(n_origin);
+  if (m0 >= M || n0 >= N) return;
+  const int m_valid = min(BM, M - m0), n_valid = min(BN, N - n0);
+
+  const uint32_t lds_base = (uint32_t)(size_t)(lds_ptr_t)smem;
+  ATile ta;
+  BTile tb;
+  ta.init(A_KC ? A + (int64_t)m0 * lda : A + m0, wave, lane, lda, m_valid, M - m0, K);
+  tb.init(B_KC ? B + (int64_t)n0 * ldb : B + n0, wave, lane, ldb, n_valid, N - n0, K);
+
+  // j-th copy instruction of this wave for the current slice (A tile's first)
+  auto issue_load = [&](int j, uint32_t stage_lds) {
+    if (j < ATile::kPerWave) ta.issue(j, stage_lds, wave);
+    else tb.issue(j - ATile::kPerWave, stage_lds + ATile::kBytes, wave);
+  };
+
+  // acc[i][j] holds the TRANSPOSE of the 16x16 block (i, j) of C: the MFMA is
+  // fed (B fragment, A fragment), so a lane ends up with 4 consecutive columns
+  // of one row of C and can store them as 8 bytes.
+  f32x4_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+
+  constexpr int KS = BK / 32;                    // K steps (32 values of K) per slice
+  constexpr int kPerStep = TM * TN;              // MFMAs per K step
+  constexpr int kMmaPerSlice = KS * kPerStep;
+  static_assert(TM + TN <= kPerStep, "interleaving plan");
+  static_assert(NW == 4, "one copy of the K loop per wave");
+  const int k_tiles = (K + BK - 1) / BK;
+  // fragments of the K step being multiplied and, filled meanwhile, of the next
+  uint4 fa[2][TM], fb[2][TN];
+
+  // K step `ks` of a slice whose first K step uses fragment buffer `par`: its
+  // MFMAs, with the TM + TN LDS reads of the next K step's fragments dealt
+  // evenly between them in the order of their first use (B0, A0, B1.., A1..),
+  // so the LDS sees a steady stream and every read has half a K step to land.
+  // (ks and par arrive as integral_constant tags: every register index below is
+  // a constant of the instantiation.)  after_mfma(q) is the caller's hook for
+  // its copy instructions.
+  auto k_step = [&](auto ks_tag, auto par_tag, const uint16_t* la, const uint16_t* lb,
+                    const uint16_t* la_next, const uint16_t* lb_next, auto&& after_mfma) {
+    constexpr int ks = decltype(ks_tag)::value, par = decltype(par_tag)::value;
+    constexpr int cur = (par + ks) & 1;
+    constexpr bool wraps = ks + 1 == KS;
+    const uint16_t* pa = wraps ? la_next : la;
+    const uint16_t* pb = wraps ? lb_next : lb;
+    constexpr int ks_pre = wraps ? 0 : ks + 1;
+    constexpr int n_reads = TM + TN;
+    static_for<kPerStep>([&](auto q_tag) {
+      constexpr int q = decltype(q_tag)::value, i = q / TN, j = q % TN;
+      acc[i][j] = Mma<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
+      // read r sits behind MFMA r * kPerStep / n_reads
+      constexpr int r = (q * n_reads + kPerStep - 1) / kPerStep;
+      if constexpr (r < n_reads && r * kPerStep / n_reads == q) {
+        if constexpr (r == 0)
+          fb[cur ^ 1][0] = BTile::frag(pb, wave_n * (BN / WN), ks_pre, lane);
+        else if constexpr (r == 1)
+          fa[cur ^ 1][0] = ATile::frag(pa, wave_m * (BM / WM), ks_pre, lane);
+        else if constexpr (r < TN + 1)
+          fb[cur ^ 1][r - 1] = BTile::frag(pb, wave_n * (BN / WN) + (r - 1) * 16, ks_pre, lane);
+        else
+          fa[cur ^ 1][r - TN] = ATile::frag(pa, wave_m * (BM / WM) + (r - TN) * 16, ks_pre, lane);
+      }
+      after_mfma(q_tag);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  if constexpr (NS == 2) {
+    // ---- two stages of 64 values of K, one barrier per slice
+    //
+    // A [row][k] operand then moves whole 128-byte lines (half as many L2
+    // requests as 64-byte pieces of rows).  Iteration kt runs the two K steps
+    // of slice kt; the barrier sits in front of the LAST one:
+    //   * by then every wave has read all fragments of slice kt (those of its
+    //     last K step during the first), so the stage is free, and has waited for
+    //     its share of slice kt+1, so that slice is published;
+    //   * the last K step prefetches the first fragments of slice kt+1 and
+    //     issues the whole copy of slice kt+2 into the freed stage, one copy
+    //     instruction every few MFMAs; the copy then has the first K step of the
+    //     next iteration (64 MFMAs) to land.
+    static_assert(KS == 2, "two K steps per slice");
+    static_assert(kLoads <= kPerStep, "at most one copy per MFMA");
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) issue_load(j, lds_base);
+    ta.advance(wave, lane);
+    tb.advance(wave, lane);
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) issue_load(j, lds_base + kStageBytes);
+    ta.advance(wave, lane);
+    tb.advance(wave, lane);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      fa[0][i] = ATile::frag(smem, wave_m * (BM / WM) + i * 16, 0, lane);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 16, 0, lane);
+
+    auto k_loop = [&](auto phase_tag) {
+      constexpr int kPhase = decltype(phase_tag)::value;
+      for (int kt = 0; kt < k_tiles; ++kt) {
+        const int stage = kt & 1;
+        const uint32_t cur_lds = lds_base + (uint32_t)stage * kStageBytes;
+        const uint16_t* la = smem + stage * kStageElems;
+        const uint16_t* lb = la + ATile::kBytes / 2;
+        const uint16_t* la_next = smem + (stage ^ 1) * kStageElems;
+        const uint16_t* lb_next = la_next + ATile::kBytes / 2;
+        static_for<KS>([&](auto ks_tag) {
+          constexpr int ks = decltype(ks_tag)::value;
+          if constexpr (ks == KS - 1) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): my reads of this stage are done
+            __syncthreads();
+          }
+          k_step(ks_tag, std::integral_constant<int, 0>{}, la, lb, la_next, lb_next,
+                 [&](auto q_tag) {
+            // copy c of slice kt+2 sits behind MFMA (c * NW + phase) * kPerStep / (kLoads * NW)
+            // of the last K step: at most one c per MFMA, found by inverting that map
+            if constexpr (ks == KS - 1) {
+              constexpr int q = decltype(q_tag)::value;
+              constexpr int c0 = (q * kLoads * NW - kPhase * kPerStep + NW * kPerStep - 1) /
+                                 (NW * kPerStep);
+              constexpr int c = c0 < 0 ? 0 : c0;
+              if constexpr (c < kLoads && (c * NW + kPhase) * kPerStep / (kLoads * NW) == q)
+                issue_load(c, cur_lds);
+            }
+          });
+          if constexpr (ks == KS - 1) {  // slice kt+2 is issued in full
+            ta.advance(wave, lane);
+            tb.advance(wave, lane);
+          }
+        });
+      }
+    };
+    switch (wave) {
+      case 0: k_loop(std::integral_constant<int, 0>{}); break;
+      case 1: k_loop(std::integral_constant<int, 1>{}); break;
+      case 2: k_loop(std::integral_constant<int, 2>{}); break;
+      default: k_loop(std::integral_constant<int, 3>{}); break;
+    }
+  } else {
+    // ---- software pipeline over the K-slices (NS LDS stages, NS >= 4)
+    //
+    // At the top of iteration kt: slices kt and kt+1 are visible to every wave,
+    // slice kt+2 is in flight, the MFMA fragments of its first K step are
+    // already in registers, and the stage of slice kt-1 is free.  The iteration
+    //   * issues the copy of slice kt+NS-1 into that free stage, one copy
+    //     instruction at a time between the MFMAs,
+    //   * runs the MFMAs of slice kt, reading the fragments of the next K step
+    //     between them; the last one prefetches the first fragments of slice
+    //     kt+1, so the MFMA pipe does not drain at the barrier,
+    //   * waits until its own share of slice kt+2 has landed and meets the other
+    //     waves at the barrier, which publishes slice kt+2 and frees stage kt.
+    // Slices past the end of K are zero-filled dummies; nothing is conditional.
+    //
+    // The barrier releases the waves of a block together, and a copy instruction
+    // keeps the CU's one address unit busy for some 16 cycles: if every wave put
+    // its copies behind the same MFMAs, each would queue behind the others and
+    // hold up its own MFMAs.  The loop therefore exists once per wave (`phase`),
+    // with the copy instructions of wave w behind MFMAs that no other wave uses;
+    // and, a slice of 32 being ONE K step, once per parity of the slice number,
+    // which names the fragment buffer in use.
+    static_assert(kLoads <= kMmaPerSlice, "at most one copy per MFMA");
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s) {
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) issue_load(j, lds_base + s * kStageBytes);
+      ta.advance(wave, lane);
+      tb.advance(wave, lane);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 3) * kLoads) : "memory");
+    __syncthreads();
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      fa[0][i] = ATile::frag(smem, wave_m * (BM / WM) + i * 16, 0, lane);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 16, 0, lane);
+
+    // one K-slice held by `stage`; parity_tag names the buffer of its first K step
+    auto slice = [&](auto phase_tag, auto parity_tag, int stage) {
+      constexpr int kPhase = decltype(phase_tag)::value;
+      const int stage_next = stage + 1 == NS ? 0 : stage + 1;
+      const int stage_free = stage == 0 ? NS - 1 : stage - 1;
+      const uint32_t free_lds = lds_base + (uint32_t)stage_free * kStageBytes;
+      const uint16_t* la = smem + stage * kStageElems;
+      const uint16_t* lb = la + ATile::kBytes / 2;
+      const uint16_t* la_next = smem + stage_next * kStageElems;
+      const uint16_t* lb_next = la_next + ATile::kBytes / 2;
+      static_for<KS>([&](auto ks_tag) {
+        k_step(ks_tag, parity_tag, la, lb, la_next, lb_next, [&](auto q_tag) {
+          // copy instruction c of phase p sits behind MFMA
+          // (c * NW + p) * kMmaPerSlice / (kLoads * NW) of the slice
+          constexpr int n = decltype(ks_tag)::value * kPerStep + decltype(q_tag)::value;
+          constexpr int c0 = (n * kLoads * NW - kPhase * kMmaPerSlice + NW * kMmaPerSlice - 1) /
+                             (NW * kMmaPerSlice);
+          constexpr int c = c0 < 0 ? 0 : c0;
+          if constexpr (c < kLoads && (c * NW + kPhase) * kMmaPerSlice / (kLoads * NW) == n)
+            issue_load(c, free_lds);
+        });
+      });
+      ta.advance(wave, lane);
+      tb.advance(wave, lane);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 3) * kLoads) : "memory");
+      __syncthreads();
+      return stage_next;
+    };
+    auto k_loop = [&](auto phase_tag) {
+      int stage = 0;
+      if constexpr (KS % 2 == 1) {
+        // two slices per trip, so that the buffer parity is fixed in the code
+        int kt = 0;
+        for (; kt + 1 < k_tiles; kt += 2) {
+          stage = slice(phase_tag, std::integral_constant<int, 0>{}, stage);
+          stage = slice(phase_tag, std::integral_constant<int, 1>{}, stage);
+        }
+        if (kt < k_tiles) stage = slice(phase_tag, std::integral_constant<int, 0>{}, stage);
+      } else {
+        for (int kt = 0; kt < k_tiles; ++kt)
+          stage = slice(phase_tag, std::integral_constant<int, 0>{}, stage);
+      }
+    };
+    switch (wave) {
+      case 0: k_loop(std::integral_constant<int, 0>{}); break;
+      case 1: k_loop(std::integral_constant<int, 1>{}); break;
+      case 2: k_loop(std::integral_constant<int, 2>{}); break;
+      default: k_loop(std::integral_constant<int, 3>{}); break;
+    }
+  }
+  // The zero-filled dummy slices are still landing in LDS: let them finish,
+  // then the whole LDS allocation is free to stage the output tile.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  // ---- epilogue: accumulator r of lane l is
+  //      C[m = l%16][n = 4*(l/16) + r] of its 16x16 block.
+  // The tile goes through LDS (row-major, rows padded by 16 bytes so that the
+  // 8-byte writes of 16 rows x 2 column groups, the 32 lanes served together,
+  // spread over the banks) and leaves as 16-byte packs: one wave instruction
+  // then stores whole 512-byte row segments.
+  const T* bias = (MODE == GEMM_FWD && g.bias)
+                      ? (const T*)g.bias + (int64_t)e * out_f : nullptr;
+  struct alignas(8) Out4 { T v[4]; };
+  constexpr int kLdc = BN + 8;   // elements per staged row
+  T* stage_c = reinterpret_cast<T*>(smem);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = wave_n * (BN / WN) + j * 16 + 4 * (lane >> 4);
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias && n0 + col < N) {
+      const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = wave_m * (BM / WM) + i * 16 + (lane & 15);
+      Out4 o;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) o.v[c] = Elem<T>::from_acc(acc[i][j][c] + bv[c]);
+      *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
+    }
+  }
+  __syncthreads();
+  // every thread moves one fixed 16-byte column pack of every kRowsPerStep-th row
+  constexpr int kRowPacks = BN / 8;                  // 16-byte packs per tile row
+  constexpr int kRowsPerStep = NT / kRowPacks;
+  constexpr int kSteps = BM / kRowsPerStep;
+  static_assert(NT % kRowPacks == 0 && BM % kRowsPerStep == 0 && kSteps <= 32,
+                "output tile must split evenly over the threads");
+  const int pk = tid % kRowPacks, r0 = tid / kRowPacks;
+  const T* sp = stage_c + r0 * kLdc + pk * 8;
+  // Rows past the expert's last one are cut off by the buffer descriptor (the
+  // bytes of this tile end with the last valid row), so the loop carries no
+  // per-row condition.
+  const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(C + (int64_t)m0 * ldc + n0), (short)0, ((m_valid - 1) * ldc + n_valid) * 2,
+      kRsrcFlags);
+  const int c_off = (r0 * ldc + pk * 8) * 2;
+  if (n0 + pk * 8 < N) {  // N is a multiple of 8: a pack is all in or all out
+    // Every pack gets registers of its own: a store holds its data registers
+    // until memory has acknowledged it, so a register reused for a later pack
+    // would make that pack wait for a full store round trip.
+    i32x4_t v[kSteps];
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u)
+      v[u] = *reinterpret_cast<const i32x4_t*>(sp + u * kRowsPerStep * kLdc);
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u)
+      __builtin_amdgcn_raw_buffer_store_b128(v[u], c_rsrc, c_off + u * kRowsPerStep * ldc * 2, 0,
+                                             0);
+  }
+}
+
+// gemm_tile() with 32x32x16 MFMAs (the wave's patch as a grid of 32x32
+// accumulators): used for DGRAD and WGRAD.
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
+__device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, TileRows where,
                                           int n_origin) {
   constexpr int NW = WM * WN;
   constexpr int NT = NW * 64;
@@ -341,10 +753,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, Til
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      fa[0][i] = ATile::frag(smem, wave_m * (BM / WM) + i * 32, 0, lane);
+      fa[0][i] = ATile::frag32(smem, wave_m * (BM / WM) + i * 32, 0, lane);
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 32, 0, lane);
+      fb[0][j] = BTile::frag32(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 32, 0, lane);
 
     auto k_loop = [&](auto phase_tag) {
       constexpr int kPhase = decltype(phase_tag)::value;
@@ -372,13 +784,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, Til
           for (int i = 0; i < TM; ++i) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-              acc[i][j] = Mma<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
+              acc[i][j] = Mma32<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
               const int q = i * TN + j;
               if (q < TM)
-                fa[cur ^ 1][q] = ATile::frag(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
+                fa[cur ^ 1][q] = ATile::frag32(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
               else if (q < TM + TN)
                 fb[cur ^ 1][q - TM] =
-                    BTile::frag(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
+                    BTile::frag32(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
               // copy instruction c of a half sits behind MFMA
               // (c * NW + phase) * kPerStep / (kHalf * NW) of its K step
               if (kk == 0 || kk == KK - 1) {
@@ -437,10 +849,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, Til
 
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      fa[0][i] = ATile::frag(smem, wave_m * (BM / WM) + i * 32, 0, lane);
+      fa[0][i] = ATile::frag32(smem, wave_m * (BM / WM) + i * 32, 0, lane);
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 32, 0, lane);
+      fb[0][j] = BTile::frag32(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 32, 0, lane);
 
     auto k_loop = [&](auto phase_tag) {
       constexpr int kPhase = decltype(phase_tag)::value;
@@ -463,13 +875,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, Til
           for (int i = 0; i < TM; ++i) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-              acc[i][j] = Mma<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
+              acc[i][j] = Mma32<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
               const int q = i * TN + j;
               if (q < TM)
-                fa[cur ^ 1][q] = ATile::frag(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
+                fa[cur ^ 1][q] = ATile::frag32(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
               else if (q < TM + TN)
                 fb[cur ^ 1][q - TM] =
-                    BTile::frag(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
+                    BTile::frag32(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
               // copy instruction c of phase p sits behind MFMA
               // (c * NW + p) * kMmaPerSlice / (kLoads * NW)
               const int n = kk * TM * TN + q;
@@ -562,6 +974,23 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, Til
   }
 }
 
+// The MFMA shape of a product: 16x16x32 where both operands are read from LDS
+// with plain 16-byte reads (FWD: 187 other instructions per 128 MFMAs), 32x32x16
+// where an operand needs the transposing read.  Measured on the cfg-4 shapes:
+// FWD 1.29-1.31 vs 1.24-1.26 PFLOP/s with 16x16x32, DGRAD 1.21 vs 1.35 and
+// WGRAD 1.24 vs 1.27 the other way round.
+#ifndef FMOE_MFMA16_MODES
+#define FMOE_MFMA16_MODES (1 << GEMM_FWD)
+#endif
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
+                                          int n_origin) {
+  if constexpr ((FMOE_MFMA16_MODES >> MODE) & 1)
+    gemm_tile16<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, where, n_origin);
+  else
+    gemm_tile32<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, where, n_origin);
+}
+
 // Remainder tiles (see the kernels below): 64 rows (the 4 waves side by side,
 // K slices of 32 in 6 LDS stages: a slice is a quarter of the MFMA work of a
 // 256-row one, so its copies need more slices of lead to cover the memory
@@ -574,7 +1003,7 @@ constexpr int kSmallStages = 6;
 // (the 4 waves side by side) that the pipeline's interleaving plan accepts.
 template <int BM, int BN, int MODE>
 constexpr bool has_small_tiles() {
-  constexpr int tm = kSmallRows / 32, tn = BN / 4 / 32;
+  constexpr int tm = kSmallRows / 32, tn = BN / 4 / 32;   // in 32x32 blocks, the tighter case
   return MODE != GEMM_WGRAD && BM > kSmallRows && BN % 128 == 0 && tm + tn <= tm * tn;
 }
 
@@ -936,8 +1365,8 @@ static int launch_mode(const GemmArgs& g, hipStream_t s) {
       // A [row][k] operand (both in FWD, dY in DGRAD) moves whole 128-byte
       // lines with K slices of 64: measured 7-8% faster for FWD, 2% for DGRAD;
       // WGRAD, with two [k][row] operands, is level with four stages of 32.
-      if (MODE != GEMM_WGRAD) return launch_cfg<T, 256, 256, 64, 2, 2, 2, MODE>(g, s);
-      return launch_cfg<T, 256, 256, 32, 2, 2, 4, MODE>(g, s);
+      if constexpr (MODE != GEMM_WGRAD) return launch_cfg<T, 256, 256, 64, 2, 2, 2, MODE>(g, s);
+      else return launch_cfg<T, 256, 256, 32, 2, 2, 4, MODE>(g, s);
     case 2: return launch_cfg<T, 128, 256, 32, 2, 2, 4, MODE>(g, s);
     case 4: return launch_cfg<T, 256, 256, 64, 2, 2, 2, MODE>(g, s);
     default: return launch_cfg<T, 128, 128, 32, 2, 2, 4, MODE>(g, s);
@@ -1013,14 +1442,22 @@ int launch_gemm_mfma_bwd(const GemmArgs& gd, const GemmArgs& gw, int dtype, hipS
   if (!gemm_mfma_supported(GEMM_DGRAD, gd, dtype) || !gemm_mfma_supported(GEMM_WGRAD, gw, dtype))
     return set_error(FMOE_ERR_UNSUPPORTED, "grouped GEMM: shape not MFMA-aligned");
   if (dtype == FMOE_BF16) return launch_bwd_t<__hip_bfloat16>(gd, gw, s);
+#ifdef FMOE_TUNING_BF16_ONLY   // tuning builds skip the f16 instantiations to compile faster
+  return set_error(FMOE_ERR_UNSUPPORTED, "tuning build: bf16 only");
+#else
   return launch_bwd_t<__half>(gd, gw, s);
+#endif
 }
 
 int launch_gemm_mfma(int mode, const GemmArgs& g, int dtype, hipStream_t s) {
   if (!gemm_mfma_supported(mode, g, dtype))
     return set_error(FMOE_ERR_UNSUPPORTED, "grouped GEMM: shape not MFMA-aligned");
   if (dtype == FMOE_BF16) return launch_t<__hip_bfloat16>(mode, g, s);
+#ifdef FMOE_TUNING_BF16_ONLY
+  return set_error(FMOE_ERR_UNSUPPORTED, "tuning build: bf16 only");
+#else
   return launch_t<__half>(mode, g, s);
+#endif
 }
 
 }  // namespace fmoe
