@@ -202,12 +202,20 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
   FMOE_REQUIRE(n_rows == 0 || dy != nullptr, FMOE_ERR_INVALID,
                "grouped_linear_bwd: dy is null");
   hipStream_t s = (hipStream_t)stream;
+  // The bf16/f16 matrix-core kernel sums the columns of dY inside its dW tiles;
+  // every other kernel leaves the bias gradient to the reduction kernel below.
+  GemmArgs gw{dy, x, dw, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
+  const bool mfma_w = dw && g_gemm_path == 0 && (n_rows == 0 || x != nullptr) &&
+                      gemm_mfma_supported(GEMM_WGRAD, gw, dtype);
+  if (mfma_w && dbias) {
+    gw.bias = dbias;
+    dbias = nullptr;  // comes out of the dW launch
+  }
   if (dx && dw && n_rows > 0 && g_gemm_path == 0) {
     FMOE_REQUIRE(w != nullptr && x != nullptr, FMOE_ERR_INVALID,
                  "grouped_linear_bwd: w or x is null");
     GemmArgs gd{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
-    GemmArgs gw{dy, x, dw, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
-    if (gemm_mfma_supported(GEMM_DGRAD, gd, dtype) && gemm_mfma_supported(GEMM_WGRAD, gw, dtype)) {
+    if (gemm_mfma_supported(GEMM_DGRAD, gd, dtype) && mfma_w) {
       rc = launch_gemm_mfma_bwd(gd, gw, dtype, s);
       if (rc) return rc;
       dx = nullptr;  // both products are under way
@@ -224,8 +232,7 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
     // runs also for n_rows == 0: experts without rows get zero gradients
     FMOE_REQUIRE(n_rows == 0 || x != nullptr, FMOE_ERR_INVALID,
                  "grouped_linear_bwd: x is null");
-    GemmArgs g{dy, x, dw, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
-    rc = run_gemm(GEMM_WGRAD, g, dtype, s);
+    rc = run_gemm(GEMM_WGRAD, gw, dtype, s);
     if (rc) return rc;
   }
   if (dbias) {

@@ -15,7 +15,9 @@ struct GemmArgs {
   const void* a;        // FWD: x      DGRAD: dy     WGRAD: dy
   const void* b;        // FWD: w      DGRAD: w      WGRAD: x
   void* c;              // FWD: y      DGRAD: dx     WGRAD: dw
-  const void* bias;     // FWD only, may be null
+  const void* bias;     // FWD: b [E, out] added to y, may be null.  WGRAD on the bf16/f16
+                        // matrix-core kernels: if not null, the [E, out] bias gradient
+                        // (column sums of dy per expert), WRITTEN by the launch
   const int32_t* seg_off;
   int64_t n_rows;       // rows allocated in the row-major activations
   int in_feat;

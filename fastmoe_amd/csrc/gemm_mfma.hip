@@ -82,6 +82,23 @@ template <> struct Mma32<__half> {
   }
 };
 
+// s + the two 16-bit values packed in `pair`, in fp32 (v_dot2 against (1, 1)).
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+template <typename T> struct ColSum;
+template <> struct ColSum<__hip_bfloat16> {
+  __device__ static __forceinline__ float add(uint32_t pair, float s) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair),
+                                           __builtin_bit_cast(bf16x2_t, 0x3f803f80u), s, false);
+  }
+};
+template <> struct ColSum<__half> {
+  __device__ static __forceinline__ float add(uint32_t pair, float s) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, pair),
+                                  __builtin_bit_cast(f16x2_t, 0x3c003c00u), s, false);
+  }
+};
+
 template <typename T> struct Mma;
 template <> struct Mma<__hip_bfloat16> {
   __device__ static __forceinline__ f32x4_t run(uint4 a, uint4 b, f32x4_t c) {
@@ -720,6 +737,25 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  // WGRAD tiles of the first column also sum the columns of their A operand
+  // (dY of this expert): the bias gradient, fp32, one v_dot2 per pair of values.
+  // g.bias then points at the [E, out_feat] gradient.
+  const bool colsum = MODE == GEMM_WGRAD && g.bias != nullptr && n0 == 0;
+  float cs[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) cs[i] = 0.f;
+  auto add_colsum = [&](const uint4 (&frags)[TM]) {
+    if (MODE == GEMM_WGRAD && colsum) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        cs[i] = ColSum<T>::add(frags[i].x, cs[i]);
+        cs[i] = ColSum<T>::add(frags[i].y, cs[i]);
+        cs[i] = ColSum<T>::add(frags[i].z, cs[i]);
+        cs[i] = ColSum<T>::add(frags[i].w, cs[i]);
+      }
+    }
+  };
+
   constexpr int KK = BK / 16;                    // MFMA K steps per slice
   constexpr int kMmaPerSlice = KK * TM * TN;
   static_assert(KK % 2 == 0, "fragment double buffer is indexed by the parity of the K step");
@@ -804,6 +840,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
               __builtin_amdgcn_sched_barrier(0);
             }
           }
+          add_colsum(fa[cur]);
           if (kk == 0) {  // slice kt+1 is issued in full: move on to slice kt+2
             ta.advance(wave, lane);
             tb.advance(wave, lane);
@@ -891,6 +928,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
               __builtin_amdgcn_sched_barrier(0);
             }
           }
+          add_colsum(fa[cur]);
         }
         ta.advance(wave, lane);
         tb.advance(wave, lane);
@@ -910,6 +948,17 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   // then the whole LDS allocation is free to stage the output tile.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+
+  // column sums: lanes l and l + 32 hold the two K halves of row l % 32
+  if (MODE == GEMM_WGRAD && colsum) {
+    T* db = (T*)const_cast<void*>(g.bias) + (int64_t)e * out_f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const float total = cs[i] + __shfl_xor(cs[i], 32, 64);
+      const int m = m0 + wave_m * (BM / WM) + i * 32 + (lane & 31);
+      if (wave_n == 0 && lane < 32 && m < M) db[m] = Elem<T>::from_acc(total);
+    }
+  }
 
   // ---- epilogue: accumulator r of lane l is
   //      C[m = l%32][n = 8*(r/4) + 4*(l/32) + r%4] of its 32x32 block.

@@ -380,22 +380,17 @@ def grouped_linear_bwd(dy: torch.Tensor, x: torch.Tensor, seg_off: torch.Tensor,
     dx = torch.empty((n, in_f), dtype=dy.dtype, device=dy.device) if need_dx else None
     dw = torch.empty_like(weight) if need_dw else None
     db = torch.empty((e, out_f), dtype=dy.dtype, device=dy.device) if need_bias else None
-    # dx and dw go down together (the library computes them in one launch where
-    # it can); the bias gradient is a call of its own so that a profile hook
-    # sees it separately
-    if need_dx and need_dw:
-        calls = (("grouped_linear_bwd", dx, dw, None), ("grouped_linear_bias_grad", None, None, db))
-    else:
-        calls = (("grouped_linear_dgrad", dx, None, None), ("grouped_linear_wgrad", None, dw, None),
-                 ("grouped_linear_bias_grad", None, None, db))
-    for name, a, b, c in calls:
-        if a is None and b is None and c is None:
-            continue
+    # one call: dX and dW go out in one launch where the library can, and on the
+    # bf16/f16 matrix-core kernels the bias gradient is summed inside the dW tiles
+    name = ("grouped_linear_bwd" if need_dx and need_dw else
+            "grouped_linear_dgrad" if need_dx else
+            "grouped_linear_wgrad" if need_dw else "grouped_linear_bias_grad")
+    if need_dx or need_dw or need_bias:
         with _launch(dy, name):
             _lib.check(
                 _L.fmoe_grouped_linear_bwd(dy.data_ptr(), x.data_ptr(),
                                            weight.data_ptr(), seg_off.data_ptr(),
-                                           _ptr(a), _ptr(b), _ptr(c), n, in_f, out_f,
+                                           _ptr(dx), _ptr(dw), _ptr(db), n, in_f, out_f,
                                            e, dt, _stream(dy)),
                 name)
     return dx, dw, db
