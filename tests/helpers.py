@@ -40,6 +40,20 @@ def max_rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
     return err / denom if denom > 0 else err
 
 
+def max_row_rel_err(got: torch.Tensor, want: torch.Tensor, floor: float = 1e-3) -> float:
+    """max over rows of (max |got - want| in the row) / (max |want| in the row):
+    the norm-wise bound of max_rel_err applied row by row (rows = the leading
+    dimension: tokens, or the experts of a weight gradient), so that a tile of
+    wrong values in a row of small magnitude cannot hide behind a large row
+    elsewhere.  Rows whose own maximum is below `floor` x the global maximum
+    are measured against that floor (a row of zeros has no scale of its own)."""
+    got = got.detach().double().cpu().reshape(got.shape[0], -1)
+    want = want.detach().double().cpu().reshape(want.shape[0], -1)
+    scale = want.abs().amax(dim=1)
+    scale = torch.clamp(scale, min=floor * max(scale.max().item(), 1e-300))
+    return ((got - want).abs().amax(dim=1) / scale).max().item()
+
+
 # tolerances: max |err| / max |ref| against a float64 evaluation of the same
 # rounded inputs.  bf16/f16: the 2e-2 bound stated for the GEMM and combine
 # outputs; f32: 1e-3 absolute in the reference's own tests

@@ -1,0 +1,272 @@
+"""The benchmark workloads themselves (bench.py's seeded cfg3, cfg4, cfg5) run as
+a whole layer, forward and backward, against the brute-force restatement of the
+reference's test oracle (tests/moe.py:30-49) on the host: all of it where the
+host can afford the arithmetic (cfg3, cfg5), a fixed sample of tokens and one
+whole expert for the Mixtral-sized cfg4.  Tolerance: the bf16 bound 2e-2, both
+norm-wise and row by row.  Also the reference-shaped dispatch (MOEScatter /
+MOEGather, module-list experts) through autograd, and nested (dict / list)
+inputs as in tests/test_mimo.py."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import DTYPES, TOL, max_rel_err, max_row_rel_err
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+ROW_TOL = 3e-2      # row-wise bound for bf16 results (2e-2 norm-wise)
+
+
+def _bench_layer(name):
+    import bench
+
+    cfg = dict(bench.CONFIGS[name], name=name)
+    layer, x, dy = bench.build_layer(cfg)
+    return cfg, layer, x, dy
+
+
+def _run_device(layer, x, dy, detach_score=False):
+    """Forward + backward on the GPU.  With detach_score the gate's scores carry
+    no gradient, so x.grad is the experts' share alone (what the oracle computes
+    when it is handed the scores as constants)."""
+    for p in layer.parameters():
+        p.grad = None
+    xd = x.detach().clone().requires_grad_(True)
+    hook = None
+    if detach_score:
+        hook = layer.gate.register_forward_hook(lambda m, a, o: (o[0], o[1].detach()))
+    try:
+        out = layer(xd)
+        out.backward(dy)
+    finally:
+        if hook is not None:
+            hook.remove()
+    torch.cuda.synchronize()
+    return out.detach(), xd.grad.detach()
+
+
+def _expert_params_cpu(layer, experts=None):
+    ex = layer.experts
+    sel = slice(None) if experts is None else experts
+    return [t.detach()[sel].float().cpu().requires_grad_(True)
+            for t in (ex.htoh4.weight, ex.htoh4.bias, ex.h4toh.weight, ex.h4toh.bias)]
+
+
+def _check(name, got, want, tol=TOL[torch.bfloat16], row_tol=ROW_TOL):
+    assert max_rel_err(got, want) <= tol, f"{name}: norm-wise"
+    assert max_row_rel_err(got, want) <= row_tol, f"{name}: row-wise"
+
+
+def _full_layer_check(name, expect_drops=False, expect_empty=0):
+    cfg, layer, x, dy = _bench_layer(name)
+    out, dx = _run_device(layer, x, dy, detach_score=True)
+    with torch.no_grad():
+        idx, score = layer.gate(x)
+    ex = layer.experts
+    counts = torch.bincount(idx[idx >= 0].view(-1), minlength=cfg["E"])
+    if expect_drops:
+        assert (idx == -1).any().item() and counts.max().item() <= layer.gate.capacity
+    assert int((counts == 0).sum()) >= expect_empty
+    cpu = _expert_params_cpu(layer)
+    x_cpu = x.float().cpu().requires_grad_(True)
+    want = O.brute_force_moe_mlp(x_cpu, idx.cpu(), score.float().cpu(), *cpu)
+    want.backward(dy.float().cpu())
+    _check("out", out, want)
+    _check("dx", dx, x_cpu.grad)
+    grads = (ex.htoh4.weight.grad, ex.htoh4.bias.grad, ex.h4toh.weight.grad, ex.h4toh.bias.grad)
+    for gname, got, ref in zip(("dW1", "db1", "dW2", "db2"), grads, cpu):
+        _check(gname, got, ref.grad)
+    # experts without rows: exactly zero gradients
+    for e in torch.nonzero(counts == 0).view(-1).tolist():
+        for got in grads:
+            assert not got[e].any().item()
+
+
+@pytest.mark.timeout(900)
+def test_config3_zipf_routing_with_capacity_full_layer():
+    """16384 tokens, d_model 2048, d_hidden 8192, 64 experts, top-2, Zipf(1.2)
+    choices clipped to 640 rows per expert: half of the expert-ordered buffers is
+    dead rows, the experts have 2.5 tiles of rows each."""
+    _full_layer_check("cfg3", expect_drops=True)
+
+
+@pytest.mark.timeout(900)
+def test_config5_fine_grained_experts_full_layer():
+    """8192 tokens, d_model 2048, d_hidden 1408, 128 experts of which 13 get no
+    token, top-8 (token-ordered scatter, tiny and empty grouped GEMMs)."""
+    _full_layer_check("cfg5", expect_empty=13)
+
+
+@pytest.mark.timeout(900)
+def test_config4_mixtral_sized_layer_on_a_sample():
+    """16384 tokens, d_model 4096, d_hidden 14336, 8 experts, top-2: 23 TFLOP per
+    step, too much for the host in full.  The oracle is evaluated on a fixed
+    sample of 384 tokens (their outputs and input gradients need nothing else)
+    and on ALL rows of one expert (its four parameter gradients need nothing
+    else); a second expert's bias gradients come from a third, cheap run."""
+    cfg, layer, x, dy = _bench_layer("cfg4")
+    out, dx = _run_device(layer, x, dy, detach_score=True)
+    with torch.no_grad():
+        idx, score = layer.gate(x)
+    idx_c, score_c = idx.cpu(), score.float().cpu()
+    ex = layer.experts
+    grads = (ex.htoh4.weight.grad, ex.htoh4.bias.grad, ex.h4toh.weight.grad, ex.h4toh.bias.grad)
+
+    # (a) a sample of tokens, all experts
+    g = torch.Generator().manual_seed(4)
+    sample = torch.randperm(cfg["T"], generator=g)[:384].sort().values
+    cpu = [t.detach().float().cpu() for t in (ex.htoh4.weight, ex.htoh4.bias,
+                                              ex.h4toh.weight, ex.h4toh.bias)]
+    xs = x[sample.cuda()].float().cpu().requires_grad_(True)
+    want = O.brute_force_moe_mlp(xs, idx_c[sample], score_c[sample], *cpu)
+    want.backward(dy[sample.cuda()].float().cpu())
+    _check("out[sample]", out[sample.cuda()], want)
+    _check("dx[sample]", dx[sample.cuda()], xs.grad)
+    del cpu
+
+    # (b) every row of one expert: its slots keep their index (renamed 0), all
+    # other slots are dropped, and the weights handed over are that expert's alone
+    for e, what in ((5, "all"),):
+        rows = torch.nonzero((idx_c == e).any(dim=1)).view(-1)
+        sub_idx = torch.where(idx_c[rows] == e, 0, -1)
+        one = _expert_params_cpu(layer, experts=slice(e, e + 1))
+        xe = x[rows.cuda()].float().cpu()
+        got = O.brute_force_moe_mlp(xe, sub_idx, score_c[rows], *one)
+        got.backward(dy[rows.cuda()].float().cpu())
+        for gname, dev, ref in zip(("dW1", "db1", "dW2", "db2"), grads, one):
+            _check(f"{gname}[{e}]", dev[e:e + 1], ref.grad)
+
+
+def _copy_fused_into_list(fused, plain):
+    plain.load_state_dict(fused.state_dict())
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_reference_shaped_route_through_autograd(dt):
+    """Module-list experts take _fmoe_general_global_forward: MOEScatter ->
+    per-expert modules -> MOEGather -> bmm.  Output, input gradient and every
+    expert's parameter gradients against the brute force, through autograd
+    (MOEScatter.backward / MOEGather.backward included), with dropped slots."""
+    from fastmoe_amd import FMoETransformerMLP
+    from fastmoe_amd.gates import GShardGate
+
+    dtype = DTYPES[dt]
+    torch.manual_seed(7)
+    fused = FMoETransformerMLP(4, 32, 64, top_k=2, gate=GShardGate)
+    plain = FMoETransformerMLP(4, 32, 64, top_k=2, gate=GShardGate, fused=False)
+    g = torch.Generator().manual_seed(8)
+    with torch.no_grad():
+        for p in fused.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * 0.3)
+    _copy_fused_into_list(fused, plain)
+    plain = plain.to(dtype).cuda()
+    plain.gate.capacity = (0.4, 0.4)            # forces drops
+    plain.gate.random_routing = False
+    x = torch.randn(150, 32, generator=g).to(dtype)
+    dy = torch.randn(150, 32, generator=g).to(dtype)
+    xd = x.cuda().requires_grad_(True)
+    hook = plain.gate.register_forward_hook(lambda m, a, o: (o[0], o[1].detach()))
+    try:
+        out = plain(xd)
+        out.backward(dy.cuda())
+    finally:
+        hook.remove()
+    with torch.no_grad():
+        idx, score = plain.gate(x.cuda())
+    assert (idx == -1).any().item()
+    names = ("htoh4.weight", "htoh4.bias", "h4toh.weight", "h4toh.bias")
+    cpu = [torch.cat([dict(e.named_parameters())[n].detach() for e in plain.experts], 0)
+           .double().cpu().requires_grad_(True) for n in names]
+    x_cpu = x.double().requires_grad_(True)
+    want = O.brute_force_moe_mlp(x_cpu, idx.cpu(), score.double().cpu(), *cpu)
+    want.backward(dy.double())
+    tol = 1e-4 if dt == "f32" else 1e-10
+    assert max_rel_err(out, want) <= tol
+    assert max_rel_err(xd.grad, x_cpu.grad) <= tol
+    for n, ref in zip(names, cpu):
+        got = torch.cat([dict(e.named_parameters())[n].grad for e in plain.experts], 0)
+        assert max_rel_err(got, ref.grad) <= tol, n
+
+
+class _TwoInputExpert(torch.nn.Module):
+    """tests/test_mimo.py:28-62: one fused expert applied to both entries of a
+    dict or list input."""
+
+    def __init__(self, num_expert, d_model, d_hidden, device_side):
+        super().__init__()
+        from fastmoe_amd import FMoELinear
+
+        self.htoh4 = FMoELinear(num_expert, d_model, d_hidden, bias=True)
+        self.h4toh = FMoELinear(num_expert, d_hidden, d_model, bias=True)
+        # with this attribute FMoE hands over a device-side SegmentTable
+        self.accepts_segment_table = device_side
+
+    def _mlp(self, t, fec):
+        return self.h4toh(F.gelu(self.htoh4(t, fec)), fec)
+
+    def forward(self, inp, fwd_expert_count):
+        if isinstance(inp, dict):
+            return {k: self._mlp(v, fwd_expert_count) for k, v in inp.items()}
+        return [self._mlp(v, fwd_expert_count) for v in inp]
+
+
+def _mimo_layer(num_expert, d_model, d_hidden, top_k, device_side):
+    from fastmoe_amd import FMoE, NaiveGate
+
+    class Gate(NaiveGate):
+        def forward(self, inp, return_all_scores=False):
+            first = inp["x"] if isinstance(inp, dict) else inp[0]
+            return super().forward(first, return_all_scores)
+
+    class Layer(FMoE):
+        def __init__(self):
+            super().__init__(num_expert=num_expert, d_model=d_model, gate=Gate, top_k=top_k)
+            self.experts = _TwoInputExpert(num_expert, d_model, d_hidden, device_side)
+
+    return Layer()
+
+
+@pytest.mark.parametrize("device_side", [False, True])
+@pytest.mark.parametrize("list_input", [False, True])
+@pytest.mark.parametrize("dt", ["f32", "f64", "f16", "bf16"])
+@pytest.mark.parametrize("num_expert,top_k", [(4, 2), (8, 3)])
+def test_nested_inputs_as_in_the_reference_mimo_suite(num_expert, top_k, dt, list_input,
+                                                      device_side):
+    """tests/test_mimo.py:100-150 (batch 4, d_model 16, d_hidden 64): a dict or
+    list of two tensors goes through the layer; both entries must agree with each
+    other (same data) and with the brute force, forward and backward, on the
+    reference-shaped route and on the device-side one."""
+    dtype = DTYPES[dt]
+    torch.manual_seed(42)
+    moe = _mimo_layer(num_expert, 16, 64, top_k, device_side)
+    with torch.no_grad():
+        for p in moe.experts.parameters():
+            p.mul_(0).add_(torch.randn(p.shape) * 0.3)
+    moe = moe.to(dtype).cuda()
+    x = torch.rand(4, 16).to(dtype)
+    a = x.cuda().requires_grad_(True)
+    b = x.cuda().requires_grad_(True)
+    inp = [a, b] if list_input else {"x": a, "y": b}
+    out = moe(inp)
+    first, second = (out[0], out[1]) if list_input else (out["x"], out["y"])
+    assert type(out) is type(inp)
+    assert torch.equal(first, second)
+    (first.float().sum() + 2 * second.float().sum()).backward()
+    with torch.no_grad():
+        idx, score = moe.gate(inp)
+    ex = moe.experts
+    cpu = [t.detach().double().cpu().requires_grad_(True)
+           for t in (ex.htoh4.weight, ex.htoh4.bias, ex.h4toh.weight, ex.h4toh.bias)]
+    x_cpu = x.double().requires_grad_(True)
+    s_cpu = score.double().cpu().requires_grad_(True)
+    want = O.brute_force_moe_mlp(x_cpu, idx.cpu(), s_cpu, *cpu)
+    (3 * want.sum()).backward()
+    tol = {"f32": 1e-4, "f64": 1e-10, "f16": 1e-2, "bf16": 4e-2}[dt]
+    assert max_rel_err(first, want) <= tol
+    for got, ref in zip((ex.htoh4.weight.grad, ex.htoh4.bias.grad, ex.h4toh.weight.grad,
+                         ex.h4toh.bias.grad), cpu):
+        assert max_rel_err(got, ref.grad) <= tol
+    # the second entry never reaches the gate: its gradient is the experts' share
+    # alone, 2/3 of what the oracle's 3 x sum() sends back to x
+    assert b.grad is not None and max_rel_err(b.grad, x_cpu.grad * (2.0 / 3.0)) <= tol
