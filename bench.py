@@ -254,6 +254,10 @@ def main():
     ap.add_argument("--config", default="cfg4", choices=sorted(CONFIGS),
                     help="workload; the default is the largest single-GPU configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--binding", default="ctypes", choices=["ctypes", "compiled"],
+                    help="Python binding of the C ABI: the ctypes module (default; carries the "
+                         "per-op event hooks the roofline figures come from) or the compiled "
+                         "pybind11 extension (whole-step timing and host enqueue time only)")
     ap.add_argument("--graph", action="store_true",
                     help="also time the same steps replayed from one HIP graph (extra field)")
     args = ap.parse_args()
@@ -263,8 +267,11 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (there is no CPU fallback of the hot path)")
 
+    if args.binding == "compiled":
+        os.environ["FMOE_BINDING"] = "compiled"
     from fastmoe_amd import fmoe_cuda
 
+    assert fmoe_cuda.BINDING == args.binding
     cfg = dict(CONFIGS[args.config], name=args.config)
     layer, x, dy = build_layer(cfg)
     x.requires_grad_(True)
@@ -304,15 +311,16 @@ def main():
     # table, and which op takes the largest share of a step.  (Every event pair
     # idles the GPU for a few microseconds, so the timed region below keeps
     # them on that one op only.)
+    hooks = args.binding == "ctypes"
     survey_steps = min(5, max(1, args.steps))
     records = []
     fmoe_cuda.profile_hook = lambda name, a, b: records.append((name, a, b))
     fmoe_cuda.profile_only = None
-    for _ in range(survey_steps):
+    for _ in range(survey_steps if hooks else 0):
         step(layer, x, dy)
     torch.cuda.synchronize()
     kernels = summarise(records, survey_steps)
-    dom = max(kernels, key=lambda n: kernels[n]["total_ms_per_step"])
+    dom = max(kernels, key=lambda n: kernels[n]["total_ms_per_step"]) if hooks else None
 
     # Timed region: exactly --steps steps, events around the dominant op only.
     records = []
@@ -328,10 +336,10 @@ def main():
     fmoe_cuda.profile_only = None
     ms_per_step = elapsed * 1e3 / args.steps
     timed = summarise(records, args.steps)
-    kernels[dom] = dict(timed[dom], timed_region=True)
-
-    kind, amount = work[dom]
-    avg_s = kernels[dom]["avg_us"] * 1e-6
+    if hooks:
+        kernels[dom] = dict(timed[dom], timed_region=True)
+    kind, amount = work[dom] if hooks else ("flop", 0.0)
+    avg_s = kernels[dom]["avg_us"] * 1e-6 if hooks else 1.0
     if kind == "flop":
         roofline = {"kernel": dom, "bound": "mfma", "achieved": round(amount / avg_s / 1e12, 2),
                     "peak": PEAK[cfg["dtype"]] / 1e12, "unit": "TFLOP/s"}
@@ -341,7 +349,9 @@ def main():
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
     traffic = MEASURED_TRAFFIC.get((args.config, dom))
     roofline["traffic"] = None if traffic is None else round(traffic)
-    roofline["avg_launch_us"] = kernels[dom]["avg_us"]
+    roofline["avg_launch_us"] = kernels[dom]["avg_us"] if hooks else None
+    if not hooks:
+        roofline = None     # no per-op events on the compiled binding
 
     result = {
         "metric": "MoE-MLP fwd+bwd tokens/s @1 MI355X",
@@ -357,6 +367,7 @@ def main():
         "vs_baseline": None,
         "dtype": cfg["dtype"],
         "data": "synthetic",
+        "binding": args.binding,
         "config": {
             "workload": (f"{args.config}: {cfg['T']} tokens, d_model {cfg['d']}, d_hidden "
                          f"{cfg['h']}, {cfg['E']} experts, top-{cfg['k']}, {cfg['dtype']}; "

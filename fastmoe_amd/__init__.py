@@ -11,13 +11,19 @@ from .linear import FMoELinear
 from .transformer import FMoETransformerMLP
 
 
-def install_as_fmoe_cuda() -> None:
+def install_as_fmoe_cuda(compiled: bool = False) -> None:
     """Registers the operator module as `fmoe_cuda`, so that the reference's
     own Python package (`import fmoe_cuda` in fmoe/functions.py:9) binds to the
-    MI355X kernels."""
+    MI355X kernels: the ctypes module, or with `compiled=True` the pybind11
+    extension of that name (cuda/fmoe_cuda.cpp:104-125 rebuilt on the C ABI)."""
     import sys
 
-    sys.modules.setdefault("fmoe_cuda", fmoe_cuda)
+    if compiled:
+        from . import _ext
+
+        sys.modules["fmoe_cuda"] = _ext.load()
+    else:
+        sys.modules.setdefault("fmoe_cuda", fmoe_cuda)
 
 
 __all__ = ["FMoE", "FMoELinear", "FMoETransformerMLP", "BaseGate", "NaiveGate",

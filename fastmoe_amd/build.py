@@ -94,5 +94,46 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
     return LIB_PATH
 
 
+EXT_DIR = os.path.join(PKG_DIR, "ext")
+EXT_SRC = os.path.join(CSRC, "fmoe_cuda_ext.cpp")
+
+
+def ext_path() -> str:
+    import sysconfig
+
+    return os.path.join(EXT_DIR, "fmoe_cuda" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_extension(verbose: bool = True) -> str:
+    """Compiles the pybind11 module `fmoe_cuda` (csrc/fmoe_cuda_ext.cpp: no
+    kernels, plain C++ against the torch headers) and links it to
+    libfmoe_hip.so, which must have been built.  Returns its path."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    os.makedirs(EXT_DIR, exist_ok=True)
+    out = ext_path()
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=fmoe_cuda",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-Wno-deprecated-declarations"]
+    cmd += ["-I" + p for p in ce.include_paths("cuda")]
+    cmd += ["-I" + sysconfig.get_paths()["include"]]
+    cmd += [EXT_SRC, "-o", out + ".tmp", "-L" + torch_lib, "-L" + LIB_DIR,
+            "-lfmoe_hip", "-ltorch_python", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10",
+            "-lc10_hip", "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath," + torch_lib]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"building the fmoe_cuda extension failed:\n{res.stderr[-4000:]}")
+    os.replace(out + ".tmp", out)
+    return out
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_extension())

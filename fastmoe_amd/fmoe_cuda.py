@@ -10,9 +10,16 @@ used by this package's own layer (``route``, ``grouped_linear_*``,
 
 Every function needs the HIP library and HIP tensors; nothing here computes
 on the CPU.
+
+Two bindings of the same C ABI exist: this module's ctypes calls (default) and
+the compiled pybind11 extension built from csrc/fmoe_cuda_ext.cpp.  With
+``FMOE_BINDING=compiled`` in the environment the operators below are replaced by
+the extension's at import time (same names and arguments; the per-op profiling
+hook is a feature of the ctypes path only).
 """
 from __future__ import annotations
 
+import os
 from typing import List, Optional, Tuple
 
 import torch
@@ -531,3 +538,18 @@ def set_gemm_path(path: int) -> None:
     library), 1 = scalar kernel only, 2..5 = matrix-core kernel with bf16/f16
     tile configuration 1..4 forced (for tests and tuning)."""
     _lib.check(_L.fmoe_set_gemm_path(path), "set_gemm_path")
+
+
+BINDING = "ctypes"
+if os.environ.get("FMOE_BINDING", "ctypes").lower() in ("compiled", "ext", "pybind"):
+    from . import _ext
+
+    _compiled = _ext.load()
+    for _name in ("expert_count", "assign_pos", "linear_forward", "linear_backward",
+                  "limit_by_capacity", "prune_gate_by_capacity", "local_scatter", "scatter_tokens",
+                  "local_gather", "route", "route_static", "grouped_linear_fwd",
+                  "grouped_linear_bwd", "gather_combine_fwd", "gather_combine_bwd",
+                  "scatter_reduce", "topk_softmax_fwd", "topk_softmax_bwd", "gelu_fwd", "gelu_bwd",
+                  "set_gemm_path", "_seg_off_from_counts"):
+        globals()[_name] = getattr(_compiled, _name)
+    BINDING = "compiled"
