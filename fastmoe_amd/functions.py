@@ -44,10 +44,17 @@ def count_by_gate(gate, num_expert, world_size, require_pos=True):
 def prepare_forward(gate, num_expert, world_size):
     """(pos, local_expert_count, global_expert_count, fwd_expert_count,
     fwd_batch_size) with the three counts on the host, as
-    fmoe/functions.py:52-75 hands them to the dispatch."""
-    pos, counts, _ = count_by_gate(gate, num_expert, world_size)
+    fmoe/functions.py:52-75 hands them to the dispatch.
+
+    ONE device-to-host copy (the E counts; the reference makes five,
+    functions.py:46,68,71-73): the number of live rows that sizes `pos` is their
+    sum, taken on the host."""
+    _single_worker(world_size)
+    with torch.no_grad():
+        pos, counts, _seg_off, _ = fmoe_cuda.route(gate.contiguous(), num_expert, want_inv=False)
     host = counts.cpu()
-    return pos, host, host, host.clone(), int(host.sum())
+    n_valid = int(host.sum())
+    return pos[:n_valid], host, host, host.clone(), n_valid
 
 
 def _local_scatter(inp, pos):

@@ -1,10 +1,11 @@
 r"""The MoE layer, mirroring fmoe/layers.py of the reference at world_size 1.
 
 `FMoE` keeps the reference's constructor and hooks.  When the experts are one
-fused module taking `(rows, fwd_expert_count)` -- this package's `_Expert` --
-the whole dispatch stays on the device: route -> scatter -> grouped GEMMs ->
-gather fused with the top-k combine, with no device-to-host copy.  Lists of
-arbitrary expert modules take the reference's route through host-side counts.
+fused module taking `(rows, fwd_expert_count)` -- this package's `_Expert` -- or
+a list of such modules (the reference's layout of FMoETransformerMLP), the whole
+dispatch stays on the device: route -> scatter -> grouped GEMMs -> gather fused
+with the top-k combine, with no device-to-host copy.  Lists of arbitrary expert
+modules take the reference's route, with ONE host read of the counts.
 """
 from __future__ import annotations
 
@@ -94,7 +95,9 @@ class FMoE(nn.Module):
     # ------------------------------------------------------------- experts
     def expert_fn(self, inp, fwd_expert_count):
         r"""Runs the experts on expert-ordered rows: the fused module in one
-        call, or each module of the list on its slice (fmoe/layers.py:164-180)."""
+        call, or each module of the list on its slice (fmoe/layers.py:164-180).
+        Arbitrary modules need real slices, hence host counts: the caller
+        (prepare_forward) has read them once."""
         if self.experts_fused:
             return self.experts(inp, fwd_expert_count)
         counts = fwd_expert_count
@@ -125,8 +128,19 @@ class FMoE(nn.Module):
 
     def _device_side_dispatch(self) -> bool:
         # the fused combine kernels keep a token's slots in the lanes of one wave
-        return (self.experts_fused and self.top_k <= 64
-                and getattr(self.experts, "accepts_segment_table", False))
+        if self.top_k > 64:
+            return False
+        if self.experts_fused:
+            return getattr(self.experts, "accepts_segment_table", False)
+        # a list of modules whose class knows how to run the whole list from a
+        # device-side segment table (this package's _Expert does)
+        can = getattr(type(self.experts[0]), "can_run_list", None) if len(self.experts) else None
+        return can is not None and can(self.experts)
+
+    def _run_experts(self, x, segments):
+        if self.experts_fused:
+            return self.experts(x, segments)
+        return type(self.experts[0]).run_list(self.experts, x, segments)
 
     # ------------------------------------------------------------- forward
     def forward(self, moe_inp):
@@ -152,7 +166,8 @@ class FMoE(nn.Module):
             plan = RoutePlan(gate_top_k_idx, self.num_expert)
             score = gate_score.reshape(-1, self.top_k)
             x = tree.map_structure(lambda t: FusedScatter.apply(t, plan), moe_inp)
-            x = self.experts(x, plan.segments)
+            x = tree.map_structure(lambda t: self._run_experts(t, plan.segments), x) \
+                if not self.experts_fused else self.experts(x, plan.segments)
             return tree.map_structure(
                 lambda t: FusedGatherCombine.apply(t, score, plan), x)
 

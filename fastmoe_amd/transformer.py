@@ -6,13 +6,47 @@ import torch.nn as nn
 
 from .functions import SegmentTable, apply_activation
 from .layers import FMoE
-from .linear import FMoELinear
+from .linear import FMoELinear, MOELinear
+
+
+class _LinearView:
+    r"""One expert of an FMoELinear as the reference's `experts[i].htoh4` would
+    look: `weight` [1, out, in] and `bias` [1, out] are views of the fused
+    parameters (gradients flow into them)."""
+
+    def __init__(self, linear: FMoELinear, i: int):
+        self.weight = linear.weight[i:i + 1]
+        self.bias = None if linear.bias is None else linear.bias[i:i + 1]
+
+    def __call__(self, inp, fwd_expert_count):
+        return MOELinear.apply(inp.type_as(self.weight), fwd_expert_count, self.weight, self.bias)
+
+
+class _ExpertView:
+    r"""`experts[i]` of a fused `_Expert`: callable like the `_Expert(1, ...)` the
+    reference keeps per expert (fmoe/transformer.py:51-55), backed by views."""
+
+    def __init__(self, parent: "_Expert", i: int):
+        self.htoh4 = _LinearView(parent.htoh4, i)
+        self.h4toh = _LinearView(parent.h4toh, i)
+        self.activation = parent.activation
+
+    def __call__(self, inp, fwd_expert_count):
+        return self.h4toh(self.activation(self.htoh4(inp, fwd_expert_count)), fwd_expert_count)
+
+    def parameters(self):
+        for lin in (self.htoh4, self.h4toh):
+            yield lin.weight
+            if lin.bias is not None:
+                yield lin.bias
 
 
 class _Expert(nn.Module):
     r"""`num_expert` two-layer MLPs held as two FMoELinear modules
     (fmoe/transformer.py:11-31).  Accepts host counts or a device-side
-    SegmentTable as `fwd_expert_count`."""
+    SegmentTable as `fwd_expert_count`.  Indexing and iterating give per-expert
+    views, so code written against the reference's list of single-expert modules
+    (`layer.experts[i].htoh4.weight`) keeps working on the fused module."""
 
     accepts_segment_table = True
 
@@ -29,6 +63,53 @@ class _Expert(nn.Module):
         x = apply_activation(self.activation, x, live)
         return self.h4toh(x, fwd_expert_count)
 
+    def __len__(self):
+        return self.htoh4.num_expert
+
+    def __getitem__(self, i):
+        n = len(self)
+        if not -n <= i < n:
+            raise IndexError(f"expert {i} of {n}")
+        return _ExpertView(self, i % n)
+
+    def __iter__(self):
+        return (_ExpertView(self, i) for i in range(len(self)))
+
+    # -- a list of such modules run as one --------------------------------------
+    @staticmethod
+    def can_run_list(experts) -> bool:
+        r"""Whether `experts` (the reference's layout: one `_Expert(1, ...)` per
+        expert) can run as ONE grouped call on concatenated weights."""
+        first = experts[0] if len(experts) else None
+        if not isinstance(first, _Expert):
+            return False
+        for e in experts:
+            if not (isinstance(e, _Expert) and e.activation is first.activation
+                    and e.htoh4.in_feat == first.htoh4.in_feat
+                    and e.htoh4.out_feat == first.htoh4.out_feat
+                    and (e.htoh4.bias is None) == (first.htoh4.bias is None)
+                    and (e.h4toh.bias is None) == (first.h4toh.bias is None)
+                    and e.htoh4.weight.dtype == first.htoh4.weight.dtype):
+                return False
+        return True
+
+    @staticmethod
+    def run_list(experts, inp, segments: SegmentTable):
+        r"""The modules of `experts` applied to their row segments in two grouped
+        GEMMs: the per-expert weights are concatenated to `[E, out, in]` for the
+        call (a copy of the weights per pass, autograd splits the gradients back),
+        and no count is read to the host."""
+        def cat(get):
+            parts = [get(e) for e in experts]
+            return None if parts[0] is None else torch.cat(parts, dim=0)
+
+        first = experts[0]
+        w1, b1 = cat(lambda e: e.htoh4.weight), cat(lambda e: e.htoh4.bias)
+        w2, b2 = cat(lambda e: e.h4toh.weight), cat(lambda e: e.h4toh.bias)
+        x = MOELinear.apply(inp.type_as(w1), segments, w1, b1)
+        x = apply_activation(first.activation, x, segments.seg_off[-1:])
+        return MOELinear.apply(x, segments, w2, b2)
+
 
 class FMoETransformerMLP(FMoE):
     r"""A complete MoE MLP block (fmoe/transformer.py:34-66).
@@ -38,9 +119,9 @@ class FMoETransformerMLP(FMoE):
     * `fused` (this build): True keeps all experts in one `_Expert` whose
       weights are `[E, out, in]` tensors and runs the device-side dispatch;
       False builds `num_expert` single-expert modules as the reference does
-      (state-dict keys `experts.<i>.htoh4.weight`), which costs a host copy of
-      the counts and a Python loop per forward.  Checkpoints in either layout
-      load into either.
+      (state-dict keys `experts.<i>.htoh4.weight`); they still run as one
+      grouped call per layer without a host read, on weights concatenated per
+      pass.  Checkpoints in either layout load into either.
     """
 
     def __init__(self, num_expert=32, d_model=1024, d_hidden=4096,

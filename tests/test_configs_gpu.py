@@ -138,28 +138,38 @@ def test_config4_mixtral_sized_layer_on_a_sample():
             _check(f"{gname}[{e}]", dev[e:e + 1], ref.grad)
 
 
-def _copy_fused_into_list(fused, plain):
-    plain.load_state_dict(fused.state_dict())
+class _PlainExpert(torch.nn.Module):
+    """A single-expert MLP like the reference's _Expert(1, ...) (fmoe/transformer.py:11-31),
+    as an ordinary module: FMoE has to slice rows for it on the host."""
+
+    def __init__(self, d_model, d_hidden=64):
+        super().__init__()
+        from fastmoe_amd import FMoELinear
+
+        self.htoh4 = FMoELinear(1, d_model, d_hidden, bias=True)
+        self.h4toh = FMoELinear(1, d_hidden, d_model, bias=True)
+
+    def forward(self, inp, fwd_expert_count):
+        return self.h4toh(F.gelu(self.htoh4(inp, fwd_expert_count)), fwd_expert_count)
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_reference_shaped_route_through_autograd(dt):
-    """Module-list experts take _fmoe_general_global_forward: MOEScatter ->
+    """Ordinary modules as experts take _fmoe_general_global_forward: MOEScatter ->
     per-expert modules -> MOEGather -> bmm.  Output, input gradient and every
     expert's parameter gradients against the brute force, through autograd
     (MOEScatter.backward / MOEGather.backward included), with dropped slots."""
-    from fastmoe_amd import FMoETransformerMLP
+    from fastmoe_amd import FMoE
     from fastmoe_amd.gates import GShardGate
 
     dtype = DTYPES[dt]
     torch.manual_seed(7)
-    fused = FMoETransformerMLP(4, 32, 64, top_k=2, gate=GShardGate)
-    plain = FMoETransformerMLP(4, 32, 64, top_k=2, gate=GShardGate, fused=False)
+    plain = FMoE(num_expert=4, d_model=32, top_k=2, gate=GShardGate, expert=_PlainExpert)
+    assert not plain._device_side_dispatch()
     g = torch.Generator().manual_seed(8)
     with torch.no_grad():
-        for p in fused.parameters():
+        for p in plain.parameters():
             p.copy_(torch.randn(p.shape, generator=g) * 0.3)
-    _copy_fused_into_list(fused, plain)
     plain = plain.to(dtype).cuda()
     plain.gate.capacity = (0.4, 0.4)            # forces drops
     plain.gate.random_routing = False
@@ -187,6 +197,134 @@ def test_reference_shaped_route_through_autograd(dt):
     for n, ref in zip(names, cpu):
         got = torch.cat([dict(e.named_parameters())[n].grad for e in plain.experts], 0)
         assert max_rel_err(got, ref.grad) <= tol, n
+
+
+class _NaiveExpert(torch.nn.Module):
+    """tests/moe.py: one Linear(d, d)."""
+
+    def __init__(self, d_model):
+        super().__init__()
+        self.linear = torch.nn.Linear(d_model, d_model)
+
+    def forward(self, x, fec=None):
+        return self.linear(x)
+
+
+class _LinearExpert(torch.nn.Module):
+    """tests/moe.py: Linear -> ReLU -> Linear."""
+
+    def __init__(self, d_model):
+        super().__init__()
+        self.model = torch.nn.Sequential(torch.nn.Linear(d_model, d_model * 2), torch.nn.ReLU(),
+                                         torch.nn.Linear(d_model * 2, d_model))
+
+    def forward(self, x, fec=None):
+        return self.model(x)
+
+
+@pytest.mark.parametrize("top_k", [2, 3])
+@pytest.mark.parametrize("experts", [[_NaiveExpert] * 4,
+                                     [_LinearExpert, _NaiveExpert] * 4])
+def test_heterogeneous_expert_modules(top_k, experts):
+    """tests/test_numerical.py:405-510 (test_fmoe_experts): a list of different
+    ordinary modules; output, input gradient and each expert's summed parameter
+    gradient against a per-token evaluation of the same modules."""
+    import copy
+
+    from fastmoe_amd import FMoE
+
+    torch.manual_seed(42)
+    moe = FMoE(num_expert=None, d_model=16, top_k=top_k, expert=experts).cuda()
+    ref_experts = copy.deepcopy(moe.experts)
+    x = torch.rand(24, 16, device="cuda")
+    a = x.clone().requires_grad_(True)
+    out = moe(a)
+    out.sum().backward()
+    with torch.no_grad():
+        idx, score = moe.gate(x)
+    b = x.clone().requires_grad_(True)
+    rows = []
+    for t in range(x.shape[0]):
+        acc = 0
+        for j in range(top_k):
+            acc = acc + score[t, j] * ref_experts[int(idx[t, j])](b[t:t + 1])[0]
+        rows.append(acc)
+    want = torch.stack(rows)
+    want.sum().backward()
+    assert max_rel_err(out, want) <= 1e-5
+
+    def grad_sums(mods):
+        return torch.stack([torch.stack([p.grad.sum() if p.grad is not None
+                                         else torch.zeros((), device="cuda")
+                                         for p in m.parameters()]).sum() for m in mods])
+
+    assert max_rel_err(grad_sums(moe.experts), grad_sums(ref_experts)) <= 1e-4
+    # the experts' share of the input gradient (the gate's own share comes on top)
+    hook = moe.gate.register_forward_hook(lambda m, i, o: (o[0], o[1].detach()))
+    try:
+        c = x.clone().requires_grad_(True)
+        moe(c).sum().backward()
+    finally:
+        hook.remove()
+    assert max_rel_err(c.grad, b.grad) <= 1e-4
+
+
+def test_module_list_of_fused_expert_class_runs_without_a_host_read():
+    """The reference's layout of FMoETransformerMLP -- one _Expert(1, ...) per
+    expert -- runs as one grouped call per layer from the device-side segment
+    table: same numbers as the fused module, gradients land on each expert's own
+    parameters, and no call of the pass synchronises with the host."""
+    from fastmoe_amd import FMoETransformerMLP
+
+    torch.manual_seed(3)
+    fused = FMoETransformerMLP(6, 64, 128, top_k=2).to(torch.bfloat16).cuda()
+    plain = FMoETransformerMLP(6, 64, 128, top_k=2, fused=False).to(torch.bfloat16).cuda()
+    plain.load_state_dict(fused.state_dict())
+    assert plain._device_side_dispatch() and len(plain.experts) == 6
+    x = torch.randn(333, 64, device="cuda", dtype=torch.bfloat16)
+    dy = torch.randn_like(x)
+    a = x.clone().requires_grad_(True)
+    fused(a).backward(dy)
+    b = x.clone().requires_grad_(True)
+    plain(b).backward(dy)                       # warm-up (tables, attributes)
+    for p in plain.parameters():
+        p.grad = None
+    b.grad = None
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("error")     # any host synchronisation raises
+    try:
+        out = plain(b)
+        out.backward(dy)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    assert torch.equal(out, fused(x))
+    assert torch.equal(b.grad, a.grad)
+    for i, e in enumerate(plain.experts):
+        assert torch.equal(e.htoh4.weight.grad[0], fused.experts.htoh4.weight.grad[i])
+        assert torch.equal(e.h4toh.bias.grad[0], fused.experts.h4toh.bias.grad[i])
+
+
+def test_fused_experts_are_indexable_like_the_reference_list():
+    """Code written against `layer.experts[i]` (fmoe/transformer.py:51-55) keeps
+    working on the fused module: views of the stacked parameters."""
+    from fastmoe_amd import FMoETransformerMLP
+
+    torch.manual_seed(4)
+    layer = FMoETransformerMLP(5, 32, 64, top_k=2).cuda()
+    ex = layer.experts
+    assert len(ex) == 5 and len(list(ex)) == 5
+    assert tuple(ex[1].htoh4.weight.shape) == (1, 64, 32) and tuple(ex[-1].h4toh.bias.shape) == (1, 32)
+    assert ex[2].htoh4.weight.data_ptr() == ex.htoh4.weight[2].data_ptr()
+    with pytest.raises(IndexError):
+        ex[5]
+    rows = torch.randn(40, 32, device="cuda")
+    counts = torch.tensor([0, 0, 0, 40, 0])
+    whole = ex(rows, counts)
+    one = ex[3](rows, torch.tensor([40]))
+    assert torch.equal(whole, one)
+    one.sum().backward()
+    assert ex.htoh4.weight.grad[3].any().item() and not ex.htoh4.weight.grad[0].any().item()
+    assert sum(p.numel() for p in ex[0].parameters()) == 64 * 32 + 64 + 32 * 64 + 32
 
 
 class _TwoInputExpert(torch.nn.Module):
