@@ -14,7 +14,6 @@ namespace fmoe {
 
 constexpr int kDispThreads = 256;
 constexpr int kDispWaves = kDispThreads / kWave;
-constexpr int kCombineUnroll = 4;   // 16-byte packs a lane of the combine kernels has in flight
 constexpr int kMaxGrid = 256 * 32;  // enough resident waves for 256 CUs
 
 __device__ __forceinline__ int64_t live_rows(int64_t n_rows,
@@ -128,18 +127,32 @@ __device__ __forceinline__ double lane_value(double v, int j) {
 // ------------------------------------------------ gather fused with combine
 // y[t] = sum_j score[t,j] * buf[inv[t,j]]; score == nullptr means weight 1
 // (the scatter backward).  VEC elements per lane per step (16 bytes, or 1).
-template <typename T, int VEC>
+//
+// SPLIT waves share a token, each taking a contiguous 1/SPLIT of the row, and a
+// lane has UNROLL packs of a source row in flight.  The host picks both so
+// that a wave holds 2 to 4 packs per lane of each row: measured on rows of
+// 8 KiB, one wave per token reaches 0.60-0.66 of the HBM peak, four waves 0.75+;
+// short rows (2 KiB) do best with one wave and 2 packs per lane.
+template <typename T, int VEC, int SPLIT, int UNROLL>
 __global__ __launch_bounds__(kDispThreads) void combine_fwd_kernel(
     const T* __restrict__ buf, const int32_t* __restrict__ inv,
     const T* __restrict__ score, T* __restrict__ y, int64_t n_tokens, int top_k,
     int64_t d) {
   using acc_t = typename Elem<T>::acc_t;
   struct alignas(sizeof(T) * VEC) Pk { T v[VEC]; };
+  constexpr int kTokPerBlock = kDispWaves / SPLIT;
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t wave = (int64_t)blockIdx.x * kDispWaves + threadIdx.x / kWave;
-  const int64_t n_waves = (int64_t)gridDim.x * kDispWaves;
+  const int w = threadIdx.x / kWave;
+  const int part = w % SPLIT;
   const int64_t row_vecs = d / VEC;
-  for (int64_t t = wave; t < n_tokens; t += n_waves) {
+  // packs [c_begin, c_end) of the row are this wave's
+  const int64_t per_part = (row_vecs + SPLIT * kWave - 1) / (SPLIT * kWave) * kWave;
+  const int64_t c_begin = part * per_part;
+  const int64_t c_end = c_begin + per_part < row_vecs ? c_begin + per_part : row_vecs;
+  const int64_t n_groups = (n_tokens + kTokPerBlock - 1) / kTokPerBlock;
+  for (int64_t tg = blockIdx.x; tg < n_groups; tg += gridDim.x) {
+    const int64_t t = tg * kTokPerBlock + w / SPLIT;
+    if (t >= n_tokens) continue;
     // lane j keeps the row and weight of slot j
     int32_t my_r = -1;
     acc_t my_s = 0;
@@ -147,12 +160,12 @@ __global__ __launch_bounds__(kDispThreads) void combine_fwd_kernel(
       my_r = inv[t * top_k + lane];
       my_s = score ? Elem<T>::to_acc(score[t * top_k + lane]) : (acc_t)1;
     }
-    // kCombineUnroll packs per lane per step: all their loads are issued
-    // before the first is used
-    for (int64_t c0 = lane; c0 < row_vecs; c0 += kWave * kCombineUnroll) {
-      acc_t acc[kCombineUnroll][VEC];
+    // UNROLL packs per lane per step: all their loads are issued before the
+    // first is used
+    for (int64_t c0 = c_begin + lane; c0 < c_end; c0 += kWave * UNROLL) {
+      acc_t acc[UNROLL][VEC];
 #pragma unroll
-      for (int u = 0; u < kCombineUnroll; ++u)
+      for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[u][v] = 0;
       for (int j = 0; j < top_k; ++j) {
@@ -162,21 +175,21 @@ __global__ __launch_bounds__(kDispThreads) void combine_fwd_kernel(
         const acc_t s = lane_value(my_s, j);
         if (r < 0) continue;
         const T* src = buf + (int64_t)r * d;
-        Pk p[kCombineUnroll];
+        Pk p[UNROLL];
 #pragma unroll
-        for (int u = 0; u < kCombineUnroll; ++u) {
+        for (int u = 0; u < UNROLL; ++u) {
           const int64_t c = c0 + (int64_t)u * kWave;
-          if (c < row_vecs) p[u] = *reinterpret_cast<const Pk*>(src + c * VEC);
+          if (c < c_end) p[u] = *reinterpret_cast<const Pk*>(src + c * VEC);
         }
 #pragma unroll
-        for (int u = 0; u < kCombineUnroll; ++u)
+        for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
           for (int v = 0; v < VEC; ++v) acc[u][v] += s * Elem<T>::to_acc(p[u].v[v]);
       }
 #pragma unroll
-      for (int u = 0; u < kCombineUnroll; ++u) {
+      for (int u = 0; u < UNROLL; ++u) {
         const int64_t c = c0 + (int64_t)u * kWave;
-        if (c < row_vecs) {
+        if (c < c_end) {
           Pk o;
 #pragma unroll
           for (int v = 0; v < VEC; ++v) o.v[v] = Elem<T>::from_acc(acc[u][v]);
@@ -188,7 +201,9 @@ __global__ __launch_bounds__(kDispThreads) void combine_fwd_kernel(
 }
 
 // dbuf[inv[i]] = score[i] * dy[i/k];  dscore[i] = <dy[i/k], buf[inv[i]]>
-template <typename T, int VEC>
+// The SPLIT waves of a token meet in LDS with their parts of the dot products
+// (summed in a fixed order: the result does not depend on timing).
+template <typename T, int VEC, int SPLIT, int UNROLL>
 __global__ __launch_bounds__(kDispThreads) void combine_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ buf,
     const int32_t* __restrict__ inv, const T* __restrict__ score,
@@ -196,44 +211,53 @@ __global__ __launch_bounds__(kDispThreads) void combine_bwd_kernel(
     int64_t d) {
   using acc_t = typename Elem<T>::acc_t;
   struct alignas(sizeof(T) * VEC) Pk { T v[VEC]; };
+  constexpr int kTokPerBlock = kDispWaves / SPLIT;
+  __shared__ acc_t part_dot[SPLIT > 1 ? kDispWaves : 1][SPLIT > 1 ? kWave : 1];
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t wave = (int64_t)blockIdx.x * kDispWaves + threadIdx.x / kWave;
-  const int64_t n_waves = (int64_t)gridDim.x * kDispWaves;
+  const int w = threadIdx.x / kWave;
+  const int part = w % SPLIT;
   const int64_t row_vecs = d / VEC;
-  for (int64_t t = wave; t < n_tokens; t += n_waves) {
+  const int64_t per_part = (row_vecs + SPLIT * kWave - 1) / (SPLIT * kWave) * kWave;
+  const int64_t c_begin = part * per_part;
+  const int64_t c_end = c_begin + per_part < row_vecs ? c_begin + per_part : row_vecs;
+  const int64_t n_groups = (n_tokens + kTokPerBlock - 1) / kTokPerBlock;
+  for (int64_t tg = blockIdx.x; tg < n_groups; tg += gridDim.x) {
+    const int64_t t = tg * kTokPerBlock + w / SPLIT;
+    const bool live = t < n_tokens;
     int32_t my_r = -1;
     acc_t my_s = 0;
-    if (lane < top_k) {
+    if (live && lane < top_k) {
       my_r = inv[t * top_k + lane];
       my_s = Elem<T>::to_acc(score[t * top_k + lane]);
     }
+    acc_t my_dot = 0;   // lane j ends up holding this wave's part of slot j's dot product
     for (int j = 0; j < top_k; ++j) {
       const int32_t r = lane_value(my_r, j);
       const acc_t s = lane_value(my_s, j);
       acc_t dot = 0;
       if (r >= 0) {
-        for (int64_t c0 = lane; c0 < row_vecs; c0 += kWave * kCombineUnroll) {
-          Pk g[kCombineUnroll], o[kCombineUnroll];
+        for (int64_t c0 = c_begin + lane; c0 < c_end; c0 += kWave * UNROLL) {
+          Pk g[UNROLL], o[UNROLL];
 #pragma unroll
-          for (int u = 0; u < kCombineUnroll; ++u) {
+          for (int u = 0; u < UNROLL; ++u) {
             const int64_t c = c0 + (int64_t)u * kWave;
-            if (c < row_vecs) {
+            if (c < c_end) {
               g[u] = *reinterpret_cast<const Pk*>(dy + t * d + c * VEC);
               o[u] = *reinterpret_cast<const Pk*>(buf + (int64_t)r * d + c * VEC);
             }
           }
 #pragma unroll
-          for (int u = 0; u < kCombineUnroll; ++u) {
+          for (int u = 0; u < UNROLL; ++u) {
             const int64_t c = c0 + (int64_t)u * kWave;
-            if (c < row_vecs) {
-              Pk w;
+            if (c < c_end) {
+              Pk wv;
 #pragma unroll
               for (int v = 0; v < VEC; ++v) {
                 const acc_t gv = Elem<T>::to_acc(g[u].v[v]);
                 dot += gv * Elem<T>::to_acc(o[u].v[v]);
-                w.v[v] = Elem<T>::from_acc(s * gv);
+                wv.v[v] = Elem<T>::from_acc(s * gv);
               }
-              *reinterpret_cast<Pk*>(dbuf + (int64_t)r * d + c * VEC) = w;
+              *reinterpret_cast<Pk*>(dbuf + (int64_t)r * d + c * VEC) = wv;
             }
           }
         }
@@ -241,7 +265,20 @@ __global__ __launch_bounds__(kDispThreads) void combine_bwd_kernel(
         for (int off = kWave / 2; off > 0; off >>= 1)
           dot += __shfl_xor(dot, off, kWave);
       }
-      if (lane == 0) dscore[t * top_k + j] = Elem<T>::from_acc(dot);
+      if (lane == j) my_dot = dot;
+    }
+    if (SPLIT == 1) {
+      if (live && lane < top_k) dscore[t * top_k + lane] = Elem<T>::from_acc(my_dot);
+    } else {
+      part_dot[w][lane] = my_dot;
+      __syncthreads();
+      if (live && part == 0 && lane < top_k) {
+        acc_t total = 0;
+#pragma unroll
+        for (int q = 0; q < SPLIT; ++q) total += part_dot[w + q][lane];
+        dscore[t * top_k + lane] = Elem<T>::from_acc(total);
+      }
+      __syncthreads();
     }
   }
 }
@@ -297,21 +334,56 @@ static int copy_unit(const void* a, const void* b, int64_t row_bytes) {
   return 1;
 }
 
+// How many waves share a token (SPLIT) and how many packs of a row a lane has
+// in flight (UNROLL) for rows of `row_vecs` packs: 2 to 4 packs per lane per wave.
+static void combine_shape(int64_t row_vecs, int* split, int* unroll) {
+  *split = row_vecs >= 8 * kWave ? 4 : (row_vecs >= 4 * kWave ? 2 : 1);
+  const int64_t per_lane = (row_vecs + *split * kWave - 1) / (*split * kWave);
+  *unroll = per_lane >= 4 ? 4 : (per_lane >= 2 ? 2 : 1);
+}
+
+static int grid_for_groups(int64_t n_tokens, int split) {
+  const int per_block = kDispWaves / split;
+  int64_t blocks = (n_tokens + per_block - 1) / per_block;
+  if (blocks < 1) blocks = 1;
+  if (blocks > kMaxGrid * 4) blocks = kMaxGrid * 4;
+  return (int)blocks;
+}
+
+#define FMOE_COMBINE_DISPATCH(KERNEL, ...)                                               \
+  do {                                                                                   \
+    if (!vec) {                                                                          \
+      hipLaunchKernelGGL((KERNEL<T, 1, 1, 4>), dim3(grid_for_groups(n_tokens, 1)),       \
+                         dim3(kDispThreads), 0, s, __VA_ARGS__);                         \
+      break;                                                                             \
+    }                                                                                    \
+    int split, unroll;                                                                   \
+    combine_shape(d / kVec, &split, &unroll);                                            \
+    const dim3 grid(grid_for_groups(n_tokens, split));                                   \
+    if (split == 4 && unroll == 4)                                                       \
+      hipLaunchKernelGGL((KERNEL<T, kVec, 4, 4>), grid, dim3(kDispThreads), 0, s, __VA_ARGS__); \
+    else if (split == 4)                                                                 \
+      hipLaunchKernelGGL((KERNEL<T, kVec, 4, 2>), grid, dim3(kDispThreads), 0, s, __VA_ARGS__); \
+    else if (split == 2 && unroll == 4)                                                  \
+      hipLaunchKernelGGL((KERNEL<T, kVec, 2, 4>), grid, dim3(kDispThreads), 0, s, __VA_ARGS__); \
+    else if (split == 2)                                                                 \
+      hipLaunchKernelGGL((KERNEL<T, kVec, 2, 2>), grid, dim3(kDispThreads), 0, s, __VA_ARGS__); \
+    else if (unroll == 4)                                                                \
+      hipLaunchKernelGGL((KERNEL<T, kVec, 1, 4>), grid, dim3(kDispThreads), 0, s, __VA_ARGS__); \
+    else if (unroll == 2)                                                                \
+      hipLaunchKernelGGL((KERNEL<T, kVec, 1, 2>), grid, dim3(kDispThreads), 0, s, __VA_ARGS__); \
+    else                                                                                 \
+      hipLaunchKernelGGL((KERNEL<T, kVec, 1, 1>), grid, dim3(kDispThreads), 0, s, __VA_ARGS__); \
+  } while (0)
+
 template <typename T>
 static int launch_combine_fwd(const void* buf, const int32_t* inv,
                               const void* score, void* y, int64_t n_tokens,
                               int top_k, int64_t d, hipStream_t s) {
   constexpr int kVec = 16 / sizeof(T);
-  const int grid = grid_for_rows(n_tokens);
   const bool vec = d % kVec == 0 && aligned(buf, 16) && aligned(y, 16);
-  if (vec)
-    hipLaunchKernelGGL((combine_fwd_kernel<T, kVec>), dim3(grid),
-                       dim3(kDispThreads), 0, s, (const T*)buf, inv,
-                       (const T*)score, (T*)y, n_tokens, top_k, d);
-  else
-    hipLaunchKernelGGL((combine_fwd_kernel<T, 1>), dim3(grid),
-                       dim3(kDispThreads), 0, s, (const T*)buf, inv,
-                       (const T*)score, (T*)y, n_tokens, top_k, d);
+  FMOE_COMBINE_DISPATCH(combine_fwd_kernel, (const T*)buf, inv, (const T*)score, (T*)y, n_tokens,
+                        top_k, d);
   FMOE_LAUNCH_CHECK("combine_fwd");
   return FMOE_OK;
 }
@@ -322,19 +394,10 @@ static int launch_combine_bwd(const void* dy, const void* buf,
                               void* dscore, int64_t n_tokens, int top_k,
                               int64_t d, hipStream_t s) {
   constexpr int kVec = 16 / sizeof(T);
-  const int grid = grid_for_rows(n_tokens);
   const bool vec = d % kVec == 0 && aligned(buf, 16) && aligned(dy, 16) &&
                    aligned(dbuf, 16);
-  if (vec)
-    hipLaunchKernelGGL((combine_bwd_kernel<T, kVec>), dim3(grid),
-                       dim3(kDispThreads), 0, s, (const T*)dy, (const T*)buf,
-                       inv, (const T*)score, (T*)dbuf, (T*)dscore, n_tokens,
-                       top_k, d);
-  else
-    hipLaunchKernelGGL((combine_bwd_kernel<T, 1>), dim3(grid),
-                       dim3(kDispThreads), 0, s, (const T*)dy, (const T*)buf,
-                       inv, (const T*)score, (T*)dbuf, (T*)dscore, n_tokens,
-                       top_k, d);
+  FMOE_COMBINE_DISPATCH(combine_bwd_kernel, (const T*)dy, (const T*)buf, inv, (const T*)score,
+                        (T*)dbuf, (T*)dscore, n_tokens, top_k, d);
   FMOE_LAUNCH_CHECK("combine_bwd");
   return FMOE_OK;
 }
