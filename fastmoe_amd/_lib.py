@@ -48,6 +48,9 @@ SIGNATURES = {
     "fmoe_grouped_linear_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p, c_int64,
                                         c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "fmoe_grouped_linear_bwd_act": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_void_p, c_int64,
+                                            c_int64, c_int64, c_int64, c_int, c_void_p]),
     "fmoe_seg_off_from_host_counts": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "fmoe_topk_softmax_fwd": (c_int, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p,
                                       c_int, c_void_p]),

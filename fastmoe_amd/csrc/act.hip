@@ -243,6 +243,19 @@ inline int direct_blocks(int64_t n) {
 }
 
 }  // namespace
+
+// Device address of the gelu'(-|x|) table of a 16-bit dtype (32768 floats,
+// indexed by the bit pattern without its sign), built on first use.
+int gelu_bwd_table(int dtype, hipStream_t s, const float** table) {
+  int cus = 0;
+  const int rc = ensure_tables(s, &cus);
+  if (rc) return rc;
+  float* base = nullptr;
+  FMOE_HIP_CHECK(hipGetSymbolAddress((void**)&base, HIP_SYMBOL(g_gelu_bwd_tab)));
+  *table = base + (dtype == FMOE_BF16 ? 0 : kTabBwd);
+  return FMOE_OK;
+}
+
 }  // namespace fmoe
 
 using namespace fmoe;

@@ -189,12 +189,13 @@ extern "C" int fmoe_grouped_linear_fwd(const void* x, const void* w,
   return run_gemm(GEMM_FWD, g, dtype, (hipStream_t)stream);
 }
 
-extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
-                                       const void* w, const int32_t* seg_off,
-                                       void* dx, void* dw, void* dbias,
-                                       int64_t n_rows, int64_t in_feat,
-                                       int64_t out_feat, int64_t n_expert,
-                                       int dtype, void* stream) {
+// Backward of the grouped linear layer; with act_pre, dx is further multiplied
+// by gelu'(act_pre): inside the DGRAD tiles' epilogue where the bf16 matrix-core
+// kernel runs, by the activation kernel over dx otherwise.
+static int linear_bwd(const void* dy, const void* x, const void* w, const int32_t* seg_off,
+                      const void* act_pre, void* dx, void* dw, void* dbias, int64_t n_rows,
+                      int64_t in_feat, int64_t out_feat, int64_t n_expert, int dtype,
+                      void* stream) {
   int rc = check_linear("grouped_linear_bwd", n_rows, in_feat, out_feat, n_expert, dtype);
   if (rc) return rc;
   FMOE_REQUIRE(seg_off != nullptr, FMOE_ERR_INVALID,
@@ -211,10 +212,18 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
     gw.bias = dbias;
     dbias = nullptr;  // comes out of the dW launch
   }
+  GemmArgs gd{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
+  void* const dx_out = dx;
+  const bool act_fused = act_pre && dx && n_rows > 0 && dtype == FMOE_BF16 && g_gemm_path == 0 &&
+                         (uintptr_t)act_pre % 16 == 0 && gemm_mfma_supported(GEMM_DGRAD, gd, dtype);
+  if (act_fused) {
+    rc = gelu_bwd_table(dtype, s, &gd.act_table);
+    if (rc) return rc;
+    gd.act_pre = act_pre;
+  }
   if (dx && dw && n_rows > 0 && g_gemm_path == 0) {
     FMOE_REQUIRE(w != nullptr && x != nullptr, FMOE_ERR_INVALID,
                  "grouped_linear_bwd: w or x is null");
-    GemmArgs gd{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
     if (gemm_mfma_supported(GEMM_DGRAD, gd, dtype) && mfma_w) {
       rc = launch_gemm_mfma_bwd(gd, gw, dtype, s);
       if (rc) return rc;
@@ -224,8 +233,7 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
   }
   if (dx && n_rows > 0) {
     FMOE_REQUIRE(w != nullptr, FMOE_ERR_INVALID, "grouped_linear_bwd: w is null");
-    GemmArgs g{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
-    rc = run_gemm(GEMM_DGRAD, g, dtype, s);
+    rc = run_gemm(GEMM_DGRAD, gd, dtype, s);
     if (rc) return rc;
   }
   if (dw) {
@@ -244,5 +252,31 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
     }
     if (rc) return rc;
   }
+  if (act_pre && !act_fused && dx_out && n_rows > 0)
+    // rows of experts only: the device-side row total is the table's last entry
+    return fmoe_gelu_bwd(dx_out, act_pre, dx_out, n_rows * in_feat, seg_off + n_expert, in_feat,
+                         dtype, stream);
   return FMOE_OK;
+}
+
+extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
+                                       const void* w, const int32_t* seg_off,
+                                       void* dx, void* dw, void* dbias,
+                                       int64_t n_rows, int64_t in_feat,
+                                       int64_t out_feat, int64_t n_expert,
+                                       int dtype, void* stream) {
+  return linear_bwd(dy, x, w, seg_off, nullptr, dx, dw, dbias, n_rows, in_feat, out_feat,
+                    n_expert, dtype, stream);
+}
+
+extern "C" int fmoe_grouped_linear_bwd_act(const void* dy, const void* x,
+                                           const void* w, const int32_t* seg_off,
+                                           const void* act_pre, void* dx, void* dw,
+                                           void* dbias, int64_t n_rows, int64_t in_feat,
+                                           int64_t out_feat, int64_t n_expert,
+                                           int dtype, void* stream) {
+  FMOE_REQUIRE(act_pre != nullptr || n_rows == 0 || dx == nullptr, FMOE_ERR_INVALID,
+               "grouped_linear_bwd_act: act_pre is null");
+  return linear_bwd(dy, x, w, seg_off, act_pre, dx, dw, dbias, n_rows, in_feat, out_feat,
+                    n_expert, dtype, stream);
 }

@@ -127,7 +127,8 @@ Tensor grouped_linear_fwd(Tensor x, Tensor seg_off, Tensor weight, OptTensor bia
 
 std::tuple<OptTensor, OptTensor, OptTensor> grouped_linear_bwd(Tensor dy, Tensor x, Tensor seg_off,
                                                                Tensor weight, bool need_bias,
-                                                               bool need_dx, bool need_dw) {
+                                                               bool need_dx, bool need_dw,
+                                                               OptTensor act_pre) {
   dev(dy, "dy");
   dev(x, "x", dy.scalar_type());
   dev(weight, "weight", dy.scalar_type());
@@ -142,7 +143,16 @@ std::tuple<OptTensor, OptTensor, OptTensor> grouped_linear_bwd(Tensor dy, Tensor
   if (need_dx) dx = torch::empty({n, in_f}, dy.options());
   if (need_dw) dw = torch::empty_like(weight);
   if (need_bias) db = torch::empty({e, out_f}, dy.options());
-  if (need_dx || need_dw || need_bias)
+  if (act_pre && need_dx) {
+    dev(*act_pre, "act_pre", dy.scalar_type());
+    need(act_pre->dim() == 2 && act_pre->size(0) == n && act_pre->size(1) == in_f,
+         "act_pre must be [rows, in]");
+    check(fmoe_grouped_linear_bwd_act(dy.data_ptr(), x.data_ptr(), weight.data_ptr(),
+                                      seg_off.data_ptr<int32_t>(), act_pre->data_ptr(), ptr(dx),
+                                      ptr(dw), ptr(db), n, in_f, out_f, e, dt(dy, "dy"),
+                                      stream_of(dy)),
+          "grouped_linear_bwd_act");
+  } else if (need_dx || need_dw || need_bias)
     check(fmoe_grouped_linear_bwd(dy.data_ptr(), x.data_ptr(), weight.data_ptr(),
                                   seg_off.data_ptr<int32_t>(), ptr(dx), ptr(dw), ptr(db), n, in_f,
                                   out_f, e, dt(dy, "dy"), stream_of(dy)),
@@ -162,7 +172,7 @@ std::vector<Tensor> linear_backward(Tensor grad_output_buf, Tensor input_buf, Te
   dev(input_buf, "input_buf", grad_output_buf.scalar_type());
   c10::DeviceGuard guard(input_buf.device());
   auto r = grouped_linear_bwd(grad_output_buf, input_buf, seg_off_from_counts(expert_count, input_buf),
-                              weight, true, true, true);
+                              weight, true, true, true, c10::nullopt);
   return {*std::get<0>(r), *std::get<1>(r), *std::get<2>(r)};
 }
 
@@ -406,7 +416,7 @@ PYBIND11_MODULE(fmoe_cuda, m) {
         py::arg("weight"), py::arg("bias") = py::none());
   m.def("grouped_linear_bwd", &grouped_linear_bwd, py::arg("dy"), py::arg("x"), py::arg("seg_off"),
         py::arg("weight"), py::arg("need_bias") = true, py::arg("need_dx") = true,
-        py::arg("need_dw") = true);
+        py::arg("need_dw") = true, py::arg("act_pre") = py::none());
   m.def("gather_combine_fwd", &gather_combine_fwd);
   m.def("gather_combine_bwd", &gather_combine_bwd);
   m.def("scatter_reduce", &scatter_reduce);

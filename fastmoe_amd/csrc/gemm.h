@@ -24,7 +24,24 @@ struct GemmArgs {
   int out_feat;
   int n_expert;
   int tile;             // 0 = choose the tile shape automatically, 1..4 = force one
+  // DGRAD on the bf16 matrix-core kernel only: if not null, dx = (dy W) * gelu'(act_pre)
+  // with act_pre [n_rows, in_feat] the pre-activations behind the layer's input,
+  // and act_table the device table of gelu'(-|x|) (gelu_bwd_table()).
+  const void* act_pre = nullptr;
+  const float* act_table = nullptr;
 };
+
+// The part of the gelu'(-|x|) table the fused DGRAD epilogue keeps in LDS: the
+// bf16 patterns of 2^-28 <= |x| < 16, 4096 floats at a fixed place behind the
+// largest staged output tile (256 rows of 256 + 8 elements).  Arguments outside
+// (zeros, denormals, |x| >= 16, infinities, NaNs) are rare in pre-activations
+// and take the full table in memory.
+constexpr int kActTabFirst = 0x3180, kActTabCount = 0x1000;
+constexpr int kActTabBytes = kActTabCount * 4;
+constexpr int kActTabLdsOffset = 256 * (256 + 8) * 2;   // bytes from the start of LDS
+
+// Device table of gelu'(-|x|) for a 16-bit dtype, built on first use (act.hip).
+int gelu_bwd_table(int dtype, hipStream_t s, const float** table);
 
 // Virtual row-tile index space of the scalar kernel: expert e owns the tiles
 // from seg_off[e] / BM + e on (the starts are strictly increasing, so tiles

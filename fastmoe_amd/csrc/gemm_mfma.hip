@@ -99,6 +99,50 @@ template <> struct ColSum<__half> {
   }
 };
 
+// dy * gelu'(x) for the two 16-bit values packed in h (dy) and p (x), rounded to
+// the storage type: what the separate activation kernel computes from its table
+// of gelu'(-|x|) (positive x: 1 - the entry).
+template <typename T> struct PackPair;
+template <> struct PackPair<__hip_bfloat16> {
+  __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+  __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+  __device__ static __forceinline__ uint32_t pack(float a, float b) {
+    return (uint32_t)__bfloat16_as_ushort(__float2bfloat16(a)) |
+           ((uint32_t)__bfloat16_as_ushort(__float2bfloat16(b)) << 16);
+  }
+};
+// f16 has 10 mantissa bits (eight times the table entries in the same range): not
+// fused, the entry point runs the separate kernel for it
+template <> struct PackPair<__half> {
+  __device__ static __forceinline__ float lo(uint32_t) { return 0.f; }
+  __device__ static __forceinline__ float hi(uint32_t) { return 0.f; }
+  __device__ static __forceinline__ uint32_t pack(float, float) { return 0u; }
+};
+// Fast form: `tab` is the slice of the table in LDS, valid for patterns whose
+// index (pattern without sign - kActTabFirst) is below kActTabCount.  The OR of
+// all indices goes into `seen`: a bit at or above kActTabCount's says that some
+// argument was outside and the result must be recomputed by the slow form (an
+// LDS read outside the slice returns whatever is there, or zero, never faults).
+template <typename T>
+__device__ __forceinline__ uint32_t gelu_bwd_pair_fast(uint32_t h, uint32_t p, const float* tab,
+                                                       uint32_t& seen) {
+  const uint32_t i0 = (p & 0x7fffu) - kActTabFirst, i1 = ((p >> 16) & 0x7fffu) - kActTabFirst;
+  seen |= i0 | i1;
+  const float n0 = tab[i0], n1 = tab[i1];
+  const float d0 = (p & 0x8000u) ? n0 : 1.f - n0;
+  const float d1 = ((int32_t)p < 0) ? n1 : 1.f - n1;
+  return PackPair<T>::pack(PackPair<T>::lo(h) * d0, PackPair<T>::hi(h) * d1);
+}
+// Slow form: any argument, from the full table in memory.
+template <typename T>
+__device__ __forceinline__ uint32_t gelu_bwd_pair_any(uint32_t h, uint32_t p,
+                                                      const float* full_tab) {
+  const float n0 = full_tab[p & 0x7fffu], n1 = full_tab[(p >> 16) & 0x7fffu];
+  const float d0 = (p & 0x8000u) ? n0 : 1.f - n0;
+  const float d1 = ((int32_t)p < 0) ? n1 : 1.f - n1;
+  return PackPair<T>::pack(PackPair<T>::lo(h) * d0, PackPair<T>::hi(h) * d1);
+}
+
 template <typename T> struct Mma;
 template <> struct Mma<__hip_bfloat16> {
   __device__ static __forceinline__ f32x4_t run(uint4 a, uint4 b, f32x4_t c) {
@@ -970,6 +1014,19 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   struct alignas(8) Out4 { T v[4]; };
   constexpr int kLdc = BN + 8;   // elements per staged row
   T* stage_c = reinterpret_cast<T*>(smem);
+  // DGRAD with the activation's backward fused in: the slice of the gelu' table
+  // goes into LDS behind the staged tile (its loads fly during the staging)
+  const bool fuse_act = MODE == GEMM_DGRAD && g.act_pre != nullptr;
+  static_assert(BM * kLdc * 2 <= kActTabLdsOffset, "the table sits behind the largest staged tile");
+  float* act_tab = reinterpret_cast<float*>(smem + kActTabLdsOffset / 2);
+  constexpr int kTabPerThread = (kActTabCount / 4 + NT - 1) / NT;
+  uint4 tab_regs[kTabPerThread];
+  if (MODE == GEMM_DGRAD && fuse_act) {
+    const uint4* src = reinterpret_cast<const uint4*>(g.act_table + kActTabFirst);
+#pragma unroll
+    for (int i = 0; i < kTabPerThread; ++i)
+      if (tid + i * NT < kActTabCount / 4) tab_regs[i] = src[tid + i * NT];
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -992,6 +1049,11 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
       }
     }
   }
+  if (MODE == GEMM_DGRAD && fuse_act) {
+#pragma unroll
+    for (int i = 0; i < kTabPerThread; ++i)
+      if (tid + i * NT < kActTabCount / 4) reinterpret_cast<uint4*>(act_tab)[tid + i * NT] = tab_regs[i];
+  }
   __syncthreads();
   // every thread moves one fixed 16-byte column pack of every kRowsPerStep-th row
   constexpr int kRowPacks = BN / 8;                  // 16-byte packs per tile row
@@ -1008,6 +1070,58 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
       (void*)(C + (int64_t)m0 * ldc + n0), (short)0, ((m_valid - 1) * ldc + n_valid) * 2,
       kRsrcFlags);
   const int c_off = (r0 * ldc + pk * 8) * 2;
+  if (MODE == GEMM_DGRAD && fuse_act) {
+    // dx = dH * gelu'(pre): the staged dH (already rounded to the storage type,
+    // as a separate activation kernel would read it) times the table value of
+    // the matching pre-activation pack, fetched through a descriptor with the
+    // tile's own bounds (a pack outside reads as zeros and its store is dropped).
+    if (n0 + pk * 8 < N) {
+      const __amdgpu_buffer_rsrc_t p_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          (void*)((const T*)g.act_pre + ((int64_t)row0 + m0) * ldc + n0), (short)0,
+          ((m_valid - 1) * ldc + n_valid) * 2, kRsrcFlags);
+      constexpr int kChunk = kSteps < 8 ? kSteps : 8;
+      constexpr int kChunks = kSteps / kChunk;
+      static_assert(kSteps % kChunk == 0, "chunks of the fused epilogue");
+      // the pre-activation packs of chunk c + 1 are in flight while chunk c is worked on
+      i32x4_t pv[2][kChunk];
+      auto load_pre = [&](auto c_tag) {
+        constexpr int c = decltype(c_tag)::value;
+#pragma unroll
+        for (int u = 0; u < kChunk; ++u)
+          pv[c & 1][u] = __builtin_amdgcn_raw_buffer_load_b128(
+              p_rsrc, c_off + (c * kChunk + u) * kRowsPerStep * ldc * 2, 0, 0);
+      };
+      load_pre(std::integral_constant<int, 0>{});
+      static_for<kChunks>([&](auto c_tag) {
+        constexpr int c = decltype(c_tag)::value;
+        if constexpr (c + 1 < kChunks) load_pre(std::integral_constant<int, c + 1>{});
+        i32x4_t hv[kChunk], ov[kChunk];
+#pragma unroll
+        for (int u = 0; u < kChunk; ++u)
+          hv[u] = *reinterpret_cast<const i32x4_t*>(sp + (c * kChunk + u) * kRowsPerStep * kLdc);
+        uint32_t seen = 0;
+#pragma unroll
+        for (int u = 0; u < kChunk; ++u)
+#pragma unroll
+          for (int wd = 0; wd < 4; ++wd)
+            ov[u][wd] = (int)gelu_bwd_pair_fast<T>((uint32_t)hv[u][wd], (uint32_t)pv[c & 1][u][wd],
+                                                   act_tab, seen);
+        if (__builtin_amdgcn_ballot_w64(seen >= (uint32_t)kActTabCount) != 0) {
+#pragma unroll
+          for (int u = 0; u < kChunk; ++u)
+#pragma unroll
+            for (int wd = 0; wd < 4; ++wd)
+              ov[u][wd] = (int)gelu_bwd_pair_any<T>((uint32_t)hv[u][wd],
+                                                    (uint32_t)pv[c & 1][u][wd], g.act_table);
+        }
+#pragma unroll
+        for (int u = 0; u < kChunk; ++u)
+          __builtin_amdgcn_raw_buffer_store_b128(
+              ov[u], c_rsrc, c_off + (c * kChunk + u) * kRowsPerStep * ldc * 2, 0, 0);
+      });
+    }
+    return;
+  }
   if (n0 + pk * 8 < N) {  // N is a multiple of 8: a pack is all in or all out
     // Every pack gets registers of its own: a store holds its data registers
     // until memory has acknowledged it, so a register reused for a later pack
@@ -1350,7 +1464,9 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   using ATile = DmaTile<BM, BK, NW, MODE != GEMM_WGRAD>;
   using BTile = DmaTile<BN, BK, NW, MODE == GEMM_FWD>;
   constexpr size_t pipe_bytes = NS * (ATile::kBytes + BTile::kBytes);
-  constexpr size_t out_bytes = (size_t)BM * (BN + 8) * 2;   // staged output tile
+  // staged output tile (+ the activation table of a fused DGRAD epilogue)
+  constexpr size_t out_bytes =
+      MODE == GEMM_DGRAD ? (size_t)kActTabLdsOffset + kActTabBytes : (size_t)BM * (BN + 8) * 2;
   constexpr size_t small_bytes = has_small_tiles<BM, BN, MODE>()
       ? (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2 : 0;
   constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
@@ -1436,7 +1552,7 @@ template <typename T, int BK, int NS>
 static int launch_bwd_fused(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
   constexpr int BM = 256, BN = 256, WM = 2, WN = 2, NT = WM * WN * 64;
   constexpr size_t pipe_bytes = (size_t)NS * (BM + BN) * BK * 2;
-  constexpr size_t out_bytes = (size_t)BM * (BN + 8) * 2;
+  constexpr size_t out_bytes = (size_t)kActTabLdsOffset + kActTabBytes;
   constexpr size_t small_bytes = (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2;
   constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
   constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;

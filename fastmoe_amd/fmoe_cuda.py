@@ -372,8 +372,13 @@ def grouped_linear_fwd(x: torch.Tensor, seg_off: torch.Tensor, weight: torch.Ten
 
 def grouped_linear_bwd(dy: torch.Tensor, x: torch.Tensor, seg_off: torch.Tensor,
                        weight: torch.Tensor, need_bias: bool = True,
-                       need_dx: bool = True, need_dw: bool = True):
-    """(dx, dw, db) of grouped_linear_fwd; entries not asked for are None."""
+                       need_dx: bool = True, need_dw: bool = True,
+                       act_pre: Optional[torch.Tensor] = None):
+    """(dx, dw, db) of grouped_linear_fwd; entries not asked for are None.
+
+    With act_pre ([rows, in], the pre-activations x = gelu(act_pre) came from) dx
+    is the gradient with respect to act_pre: the backward of the activation is
+    applied to it, inside the kernel's epilogue where the library can."""
     _dev(dy, "dy")
     _dev(x, "x", dy.dtype)
     _dev(weight, "weight", dy.dtype)
@@ -392,7 +397,17 @@ def grouped_linear_bwd(dy: torch.Tensor, x: torch.Tensor, seg_off: torch.Tensor,
     name = ("grouped_linear_bwd" if need_dx and need_dw else
             "grouped_linear_dgrad" if need_dx else
             "grouped_linear_wgrad" if need_dw else "grouped_linear_bias_grad")
-    if need_dx or need_dw or need_bias:
+    if act_pre is not None and need_dx:
+        _dev(act_pre, "act_pre", dy.dtype)
+        _need(tuple(act_pre.shape) == (n, in_f), "act_pre must be [rows, in]")
+        with _launch(dy, name):     # same kernels and FLOPs as without act_pre: same op name
+            _lib.check(
+                _L.fmoe_grouped_linear_bwd_act(dy.data_ptr(), x.data_ptr(),
+                                               weight.data_ptr(), seg_off.data_ptr(),
+                                               act_pre.data_ptr(), _ptr(dx), _ptr(dw),
+                                               _ptr(db), n, in_f, out_f, e, dt, _stream(dy)),
+                name)
+    elif need_dx or need_dw or need_bias:
         with _launch(dy, name):
             _lib.check(
                 _L.fmoe_grouped_linear_bwd(dy.data_ptr(), x.data_ptr(),

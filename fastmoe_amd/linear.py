@@ -8,7 +8,7 @@ import torch.nn as nn
 from torch.autograd import Function
 
 from . import fmoe_cuda
-from .functions import SegmentTable
+from .functions import SegmentTable, apply_activation
 
 
 def _segments(fwd_expert_count, device) -> torch.Tensor:
@@ -41,6 +41,51 @@ class MOELinear(Function):
             grad_out.contiguous(), x, seg_off, weight.contiguous(),
             need_bias=need_db, need_dx=need_dx, need_dw=need_dw)
         return dx, None, dw, db
+
+
+class MOEGeluLinear(Function):
+    r"""`linear(gelu(pre))` as one autograd node: the activation between the two
+    expert layers and the second layer (fmoe/transformer.py:28-31 for
+    torch.nn.GELU()).  Forward runs the activation kernel and the grouped GEMM;
+    backward hands the saved pre-activations to the grouped backward, which
+    applies gelu' to dX inside the GEMM epilogue (bf16) instead of writing
+    dY W to memory for a separate activation kernel to read back."""
+
+    @staticmethod
+    def forward(ctx, pre, fwd_expert_count, weight, bias=None):
+        pre = pre.contiguous()
+        seg_off = _segments(fwd_expert_count, pre.device)
+        act = fmoe_cuda.gelu_fwd(pre, seg_off[-1:])      # rows past the last segment are dead
+        out = fmoe_cuda.grouped_linear_fwd(act, seg_off, weight.contiguous(),
+                                           None if bias is None else bias.contiguous())
+        ctx.save_for_backward(pre, act, seg_off, weight, bias)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (pre, act, seg_off, weight, bias) = ctx.saved_tensors
+        need_dx, _, need_dw, need_db = ctx.needs_input_grad
+        need_db = need_db and torch.is_tensor(bias)
+        dpre, dw, db = fmoe_cuda.grouped_linear_bwd(
+            grad_out.contiguous(), act, seg_off, weight.contiguous(),
+            need_bias=need_db, need_dx=need_dx, need_dw=need_dw, act_pre=pre)
+        return dpre, None, dw, db
+
+
+def is_exact_gelu(activation, x: torch.Tensor) -> bool:
+    r"""Whether `activation(x)` is the erf GELU the library has kernels for."""
+    return (type(activation) is torch.nn.GELU
+            and getattr(activation, "approximate", "none") == "none" and x.is_cuda
+            and x.dtype in (torch.float32, torch.float64, torch.float16, torch.bfloat16))
+
+
+def act_linear(activation, pre, fwd_expert_count, weight, bias):
+    r"""`linear(activation(pre))` over the experts' row segments."""
+    if is_exact_gelu(activation, pre) and pre.dtype == weight.dtype:
+        return MOEGeluLinear.apply(pre, fwd_expert_count, weight, bias)
+    live = fwd_expert_count.seg_off[-1:] if isinstance(fwd_expert_count, SegmentTable) else None
+    x = apply_activation(activation, pre, live)
+    return MOELinear.apply(x.type_as(weight), fwd_expert_count, weight, bias)
 
 
 class FMoELinear(nn.Module):

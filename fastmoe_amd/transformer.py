@@ -4,9 +4,9 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .functions import SegmentTable, apply_activation
+from .functions import SegmentTable
 from .layers import FMoE
-from .linear import FMoELinear, MOELinear
+from .linear import FMoELinear, MOELinear, act_linear
 
 
 class _LinearView:
@@ -58,10 +58,10 @@ class _Expert(nn.Module):
 
     def forward(self, inp, fwd_expert_count):
         x = self.htoh4(inp, fwd_expert_count)
-        # with a device-side segment table, the activation skips the dead rows
-        live = fwd_expert_count.seg_off[-1:] if isinstance(fwd_expert_count, SegmentTable) else None
-        x = apply_activation(self.activation, x, live)
-        return self.h4toh(x, fwd_expert_count)
+        # activation and second layer as one node: the activation's backward runs
+        # inside the second layer's backward kernel
+        return act_linear(self.activation, x, fwd_expert_count, self.h4toh.weight,
+                          self.h4toh.bias)
 
     def __len__(self):
         return self.htoh4.num_expert
@@ -107,8 +107,7 @@ class _Expert(nn.Module):
         w1, b1 = cat(lambda e: e.htoh4.weight), cat(lambda e: e.htoh4.bias)
         w2, b2 = cat(lambda e: e.h4toh.weight), cat(lambda e: e.h4toh.bias)
         x = MOELinear.apply(inp.type_as(w1), segments, w1, b1)
-        x = apply_activation(first.activation, x, segments.seg_off[-1:])
-        return MOELinear.apply(x, segments, w2, b2)
+        return act_linear(first.activation, x, segments, w2, b2)
 
 
 class FMoETransformerMLP(FMoE):

@@ -248,6 +248,24 @@ int fmoe_grouped_linear_bwd(const void* dy, const void* x, const void* w,
                             void* stream);
 
 /*
+ * fmoe_grouped_linear_bwd for a layer whose input is act = gelu(act_pre), with
+ * the activation's backward folded in: dx = (dY[seg_e] * W_e) .* gelu'(act_pre),
+ * x being act (dW is unchanged).  act_pre is [n_rows, in_feat].  bf16 on the
+ * matrix-core kernel applies the factor in the tile epilogue, so the product
+ * dY * W never reaches memory; every other case runs fmoe_gelu_bwd over dx, with
+ * the same bits out.  The first bf16 call builds the activation tables (see
+ * fmoe_gelu_fwd).
+ * Replaces, for the second linear layer of an expert, fmoe_cuda.linear_backward
+ * followed by the backward of the activation in between
+ * (fmoe/transformer.py:25-33: htoh4 -> activation -> h4toh).
+ */
+int fmoe_grouped_linear_bwd_act(const void* dy, const void* x, const void* w,
+                                const int32_t* seg_off, const void* act_pre,
+                                void* dx, void* dw, void* dbias, int64_t n_rows,
+                                int64_t in_feat, int64_t out_feat,
+                                int64_t n_expert, int dtype, void* stream);
+
+/*
  * seg_off (device int32[E+1]) from HOST int64 counts, the form in which the
  * reference passes counts to its linear ops (cuda/parallel_linear.cuh:69-70
  * dereferences expert_count on the host).  `seg_off` must stay alive until
