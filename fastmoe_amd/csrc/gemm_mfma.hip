@@ -177,10 +177,13 @@ struct DmaTile {
   static constexpr int kRowPacks = R / 8;           // packs per [k] row (KC == false)
   static constexpr int kKPacks = BK / 8;            // packs per [row] row (KC == true)
 
-  // XOR applied to the pack index of a [row][BK] row so that 16 consecutive
-  // rows read at the same K offset cover all 64 LDS banks.
+  // XOR applied to the pack index of a [row][BK] row.  Chosen by timing
+  // ds_read_b128 with four waves reading at once, over all XOR maps that are
+  // linear in the row's bits: these two serve both fragment shapes at the full
+  // LDS rate (16 rows x 4 packs per instruction for the 16x16x32 MFMA, 32 rows x
+  // 2 packs for 32x32x16); without them the reads take two to four times as long.
   __device__ static __forceinline__ int row_swizzle(int row) {
-    return BK == 64 ? ((row & 7) ^ ((row >> 3) & 1)) : ((row >> 2) & 3);
+    return BK == 64 ? ((row >> 1) & 7) : (((row >> 4) & 1) | (((row >> 2) & 1) << 1));
   }
   // K offset (elements) inside the slice of the pack lane `lane` copies in
   // block b (KC only).
@@ -448,9 +451,12 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   // (ks and par arrive as integral_constant tags: every register index below is
   // a constant of the instantiation.)  after_mfma(q) is the caller's hook for
   // its copy instructions.
-  auto k_step = [&](auto ks_tag, auto par_tag, const uint16_t* la, const uint16_t* lb,
-                    const uint16_t* la_next, const uint16_t* lb_next, auto&& after_mfma) {
+  auto k_step = [&](auto ks_tag, auto par_tag, auto bunch_tag, const uint16_t* la,
+                    const uint16_t* lb, const uint16_t* la_next, const uint16_t* lb_next,
+                    auto&& after_mfma) {
     constexpr int ks = decltype(ks_tag)::value, par = decltype(par_tag)::value;
+    // bunched: read r right behind MFMA r, so that all are on their way early
+    constexpr bool bunched = decltype(bunch_tag)::value;
     constexpr int cur = (par + ks) & 1;
     constexpr bool wraps = ks + 1 == KS;
     const uint16_t* pa = wraps ? la_next : la;
@@ -460,9 +466,9 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
     static_for<kPerStep>([&](auto q_tag) {
       constexpr int q = decltype(q_tag)::value, i = q / TN, j = q % TN;
       acc[i][j] = Mma<T>::run(fb[cur][j], fa[cur][i], acc[i][j]);
-      // read r sits behind MFMA r * kPerStep / n_reads
-      constexpr int r = (q * n_reads + kPerStep - 1) / kPerStep;
-      if constexpr (r < n_reads && r * kPerStep / n_reads == q) {
+      // read r sits behind MFMA r * kPerStep / n_reads (or behind MFMA r)
+      constexpr int r = bunched ? q : (q * n_reads + kPerStep - 1) / kPerStep;
+      if constexpr (r < n_reads && (bunched || r * kPerStep / n_reads == q)) {
         if constexpr (r == 0)
           fb[cur ^ 1][0] = BTile::frag(pb, wave_n * (BN / WN), ks_pre, lane);
         else if constexpr (r == 1)
@@ -478,20 +484,30 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   };
 
   if constexpr (NS == 2) {
-    // ---- two stages of 64 values of K, one barrier per slice
+    // ---- two stages of 64 values of K, two barriers per slice
     //
     // A [row][k] operand then moves whole 128-byte lines (half as many L2
     // requests as 64-byte pieces of rows).  Iteration kt runs the two K steps
-    // of slice kt; the barrier sits in front of the LAST one:
-    //   * by then every wave has read all fragments of slice kt (those of its
-    //     last K step during the first), so the stage is free, and has waited for
-    //     its share of slice kt+1, so that slice is published;
-    //   * the last K step prefetches the first fragments of slice kt+1 and
-    //     issues the whole copy of slice kt+2 into the freed stage, one copy
-    //     instruction every few MFMAs; the copy then has the first K step of the
-    //     next iteration (64 MFMAs) to land.
+    // of slice kt out of registers filled one K step ahead:
+    //   * the first K step reads the fragments of the second one right away, one
+    //     read behind each of its first MFMAs.  When they have landed the stage of
+    //     slice kt is not needed any more; the waves say so at the first barrier
+    //     (behind MFMA kFreeAt - 1) and start copying slice kt+2 into it;
+    //   * the copies are dealt over the rest of the slice, one copy of the block
+    //     every (kCopyEnd - kFreeAt) / (4 kLoads) MFMAs: the CU's one address unit
+    //     takes about 20 cycles per copy (52 bytes per cycle measured), so the 64
+    //     copies of a 256 x 256 slice keep it busy for 60 % of the slice's MFMA
+    //     time and must not be packed into one K step, where the waves would wait
+    //     at every copy for the unit to take it;
+    //   * the second barrier, in front of the last K step, publishes slice kt+1
+    //     (copied during the slice before, landed by now); the last K step reads
+    //     the first fragments of slice kt+1 between its MFMAs.
     static_assert(KS == 2, "two K steps per slice");
-    static_assert(kLoads <= kPerStep, "at most one copy per MFMA");
+    // first MFMA of a slice behind which copies may go, and the MFMA the last
+    // one has gone before (the slice has 2 * kPerStep MFMAs)
+    constexpr int kFreeAt = TM + TN + 8, kCopyEnd = 2 * kPerStep - 4;
+    static_assert(kFreeAt < kPerStep && kLoads <= kCopyEnd - kFreeAt,
+                  "at most one copy per MFMA of a wave");
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) issue_load(j, lds_base);
     ta.advance(wave, lane);
@@ -509,8 +525,18 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
     for (int j = 0; j < TN; ++j)
       fb[0][j] = BTile::frag(smem + ATile::kBytes / 2, wave_n * (BN / WN) + j * 16, 0, lane);
 
+    // MFMA (counted through the slice) behind which copy c of the wave in
+    // position `phase` goes: the 4 * kLoads copies of the block are dealt evenly
+    // over MFMAs kFreeAt .. kCopyEnd - 1, one wave after the other.
     auto k_loop = [&](auto phase_tag) {
       constexpr int kPhase = decltype(phase_tag)::value;
+      // copies of this wave issued before MFMA n of the slice
+      auto issued_before = [](int n) constexpr {
+        int cnt = 0;
+        for (int c = 0; c < kLoads; ++c)
+          if (kFreeAt + (c * NW + kPhase) * (kCopyEnd - kFreeAt) / (kLoads * NW) < n) ++cnt;
+        return cnt;
+      };
       for (int kt = 0; kt < k_tiles; ++kt) {
         const int stage = kt & 1;
         const uint32_t cur_lds = lds_base + (uint32_t)stage * kStageBytes;
@@ -521,20 +547,25 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
         static_for<KS>([&](auto ks_tag) {
           constexpr int ks = decltype(ks_tag)::value;
           if constexpr (ks == KS - 1) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): my reads of this stage are done
+            // slice kt+1 is needed from here on: everything but the copies of slice
+            // kt+2 issued so far has landed
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(issued_before(kPerStep)) : "memory");
             __syncthreads();
           }
-          k_step(ks_tag, std::integral_constant<int, 0>{}, la, lb, la_next, lb_next,
+          k_step(ks_tag, std::integral_constant<int, 0>{},
+                 std::integral_constant<bool, ks == 0>{}, la, lb, la_next, lb_next,
                  [&](auto q_tag) {
-            // copy c of slice kt+2 sits behind MFMA (c * NW + phase) * kPerStep / (kLoads * NW)
-            // of the last K step: at most one c per MFMA, found by inverting that map
-            if constexpr (ks == KS - 1) {
-              constexpr int q = decltype(q_tag)::value;
-              constexpr int c0 = (q * kLoads * NW - kPhase * kPerStep + NW * kPerStep - 1) /
-                                 (NW * kPerStep);
-              constexpr int c = c0 < 0 ? 0 : c0;
-              if constexpr (c < kLoads && (c * NW + kPhase) * kPerStep / (kLoads * NW) == q)
+            constexpr int n = ks * kPerStep + decltype(q_tag)::value;
+            if constexpr (n == kFreeAt - 1) {
+              // the fragments of the slice's last K step are in registers (or on
+              // their way: wait for them): once every wave says so, the stage is free
+              __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+              __syncthreads();
+            }
+            if constexpr (n >= kFreeAt && n < kCopyEnd) {
+              constexpr int c = issued_before(n);   // the next copy to issue
+              if constexpr (c < kLoads &&
+                            kFreeAt + (c * NW + kPhase) * (kCopyEnd - kFreeAt) / (kLoads * NW) == n)
                 issue_load(c, cur_lds);
             }
           });
@@ -602,7 +633,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
       const uint16_t* la_next = smem + stage_next * kStageElems;
       const uint16_t* lb_next = la_next + ATile::kBytes / 2;
       static_for<KS>([&](auto ks_tag) {
-        k_step(ks_tag, parity_tag, la, lb, la_next, lb_next, [&](auto q_tag) {
+        k_step(ks_tag, parity_tag, std::false_type{}, la, lb, la_next, lb_next, [&](auto q_tag) {
           // copy instruction c of phase p sits behind MFMA
           // (c * NW + p) * kMmaPerSlice / (kLoads * NW) of the slice
           constexpr int n = decltype(ks_tag)::value * kPerStep + decltype(q_tag)::value;
