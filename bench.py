@@ -51,15 +51,18 @@ CONFIGS = {
 DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 PEAK = {"hbm": 8.0e12, "bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 
-# HBM bytes per launch (read + write) from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# counter runs of this script, scaled by what the same counters read for the
-# row-scatter kernel, whose traffic is known (factors 1.035 and 1.000).  Only
-# the workloads that were measured have an entry.
+# Bytes per launch (read + write) that leave L2 towards the Infinity Cache and
+# HBM, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script, scaled
+# by what the same counters read in the same run for the row-scatter kernel,
+# whose traffic is known (FETCH_SIZE x 1.035 on cfg2 and cfg5, x 0.998 on cfg4;
+# WRITE_SIZE x 1.000).  Only the workloads that were measured have an entry.
 MEASURED_TRAFFIC = {
-    ("cfg2", "grouped_linear_bwd"): (273.9 + 208.0) * 2 ** 20,
-    ("cfg2", "grouped_linear_fwd"): (153.7 + 80.0) * 2 ** 20,
-    ("cfg5", "grouped_linear_bwd"): (1185.5 + 920.0) * 2 ** 20,
-    ("cfg5", "grouped_linear_fwd"): (808.7 + 216.0) * 2 ** 20,
+    ("cfg2", "grouped_linear_bwd"): (308.8 + 220.2) * 2 ** 20,
+    ("cfg2", "grouped_linear_fwd"): (153.8 + 80.0) * 2 ** 20,
+    ("cfg4", "grouped_linear_bwd"): (5920.3 + 1550.9) * 2 ** 20,
+    ("cfg4", "grouped_linear_fwd"): (2908.6 + 576.0) * 2 ** 20,
+    ("cfg5", "grouped_linear_bwd"): (1240.5 + 951.4) * 2 ** 20,
+    ("cfg5", "grouped_linear_fwd"): (813.2 + 216.0) * 2 ** 20,
 }
 
 
