@@ -39,6 +39,7 @@
 // Operand roles follow cuda/parallel_linear.cuh:69-87,124-147 of the
 // reference; the per-expert cuBLAS loop there becomes a tile index space.
 #include <type_traits>
+#include <algorithm>
 #include <utility>
 
 #include "dma_desc.h"
@@ -371,7 +372,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   constexpr bool B_KC = MODE == GEMM_FWD;
   constexpr int TM = BM / WM / 16, TN = BN / WN / 16;   // 16x16 blocks of a wave
   static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0 && BK % 32 == 0, "tile shape");
-  static_assert((NS >= 4 && NS <= 6) || (NS == 2 && BK == 64), "LDS stages");
+  static_assert((NS >= 4 && NS <= 8) || (NS == 2 && BK == 64), "LDS stages");
   using ATile = DmaTile<BM, BK, NW, A_KC>;
   using BTile = DmaTile<BN, BK, NW, B_KC>;
   constexpr int kStageBytes = ATile::kBytes + BTile::kBytes;
@@ -748,7 +749,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   constexpr bool B_KC = MODE == GEMM_FWD;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % 16 == 0, "tile shape");
-  static_assert((NS >= 4 && NS <= 6) || (NS == 2 && BK == 64), "LDS stages");
+  static_assert((NS >= 4 && NS <= 8) || (NS == 2 && BK == 64), "LDS stages");
   using ATile = DmaTile<BM, BK, NW, A_KC>;
   using BTile = DmaTile<BN, BK, NW, B_KC>;
   constexpr int kStageBytes = ATile::kBytes + BTile::kBytes;
@@ -834,7 +835,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   constexpr int KK = BK / 16;                    // MFMA K steps per slice
   constexpr int kMmaPerSlice = KK * TM * TN;
   static_assert(KK % 2 == 0, "fragment double buffer is indexed by the parity of the K step");
-  static_assert(TM + TN <= TM * TN, "interleaving plan");
+  static_assert(NS != 2 || TM + TN <= TM * TN, "interleaving plan of the two-stage loop");
   static_assert(NW == 4, "one copy of the K loop per wave");
   const int k_tiles = (K + BK - 1) / BK;
   uint4 fa[2][TM], fb[2][TN];
@@ -1002,6 +1003,15 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
                 if ((c * NW + kPhase) * kMmaPerSlice / (kLoads * NW) == n) issue_load(c, free_lds);
               __builtin_amdgcn_sched_barrier(0);
             }
+          }
+          // narrow wave tiles have fewer MFMAs per K step than fragments to read
+#pragma unroll
+          for (int q = TM * TN; q < TM + TN; ++q) {
+            if (q < TM)
+              fa[cur ^ 1][q] = ATile::frag32(pa, wave_m * (BM / WM) + q * 32, kk_pre, lane);
+            else
+              fb[cur ^ 1][q - TM] =
+                  BTile::frag32(pb, wave_n * (BN / WN) + (q - TM) * 32, kk_pre, lane);
           }
           add_colsum(fa[cur]);
         }
@@ -1241,10 +1251,38 @@ __device__ __forceinline__ void edge_aware_tile(const GemmArgs& g, uint16_t* sme
   gemm_tile<T, BM, BN, BK, WM, WN, NS, MODE>(g, smem, where, n0);
 }
 
-// Runs the remainder tile at rows [where.m0, where.cnt) of its expert.
+// A remainder tile streams its whole weight strip (BN columns x K) through one
+// CU for 64 rows of output, at the rate of that CU's address unit (~52 bytes per
+// cycle): when a launch has so few of them that they would leave most CUs idle
+// (at most kNarrowMax; cfg 2 has 32 to 128 behind 1024 full tiles) they are cut
+// into narrower ones, 64 columns for FWD and 128 for DGRAD (whose weight tile is
+// [k][columns] and needs 128 of them for its LDS layout): four or two times as
+// many CUs then share the streaming.  It pays from K = 2048 on (measured on the
+// cfg-2 shapes from cold caches: K = 4096 forward 209 -> 180 us, dX 199 -> 182 us;
+// at K = 1024 the fixed cost of four times as many tiles eats the gain).
+constexpr int kNarrowMax = 128;
+constexpr int kNarrowMinK = 2048;
+template <int BM, int BN, int MODE>
+constexpr int narrow_factor() {
+  return (BM == 256 && BN == 256 && MODE != GEMM_WGRAD) ? (MODE == GEMM_FWD ? 4 : 2) : 1;
+}
+
+// Runs the remainder tile at rows [where.m0, where.cnt) of its expert; n_tile
+// counts columns in units of BN, or of BN / narrow_factor for narrow tiles.
 template <typename T, int BM, int BN, int MODE>
 __device__ __forceinline__ void remainder_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
-                                               int n_tile) {
+                                               int n_tile, bool narrow) {
+  constexpr int kF = narrow_factor<BM, BN, MODE>();
+  if constexpr (kF > 1) {
+    if (narrow) {
+      constexpr int NB = BN / kF;
+      if (where.cnt - where.m0 > kSmallRows)
+        gemm_tile<T, 2 * kSmallRows, NB, kSmallBK, 2, 2, 4, MODE>(g, smem, where, n_tile * NB);
+      else
+        gemm_tile<T, kSmallRows, NB, kSmallBK, 2, 2, 8, MODE>(g, smem, where, n_tile * NB);
+      return;
+    }
+  }
   if constexpr (BM >= 4 * kSmallRows) {
     if (where.cnt - where.m0 > kSmallRows) {
       gemm_tile<T, 2 * kSmallRows, BN, kSmallBK, 2, 2, 4, MODE>(g, smem, where, n_tile * BN);
@@ -1417,18 +1455,23 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   }
   RowTiles<BM, kSmall, NW> rows;
   rows.scan(g.seg_off, g.n_expert, s_wave_sum);
-  const int live_f = rows.rows_f * tiles_n, live = live_f + rows.rows_s * tiles_n;
+  constexpr int kF = kSmall ? narrow_factor<BM, BN, MODE>() : 1;
+  const int wide_s = rows.rows_s * tiles_n;
+  const bool narrow = kF > 1 && wide_s <= kNarrowMax &&
+                      (MODE == GEMM_FWD ? g.in_feat : g.out_feat) >= kNarrowMinK;
+  const int cols_s = narrow ? tiles_n * kF : tiles_n;
+  const int live_f = rows.rows_f * tiles_n, live = live_f + rows.rows_s * cols_s;
   if (live == 0) return;
   const int t = tile_number(pid, live);
   if (t >= live) return;  // the same for the whole block
   const bool small = t >= live_f;  // BM-row tiles start first: they take longer
   int v, n_tile;
-  if (small) tile_order(t - live_f, rows.rows_s, tiles_n, v, n_tile);
+  if (small) tile_order(t - live_f, rows.rows_s, cols_s, v, n_tile);
   else tile_order(t, rows.rows_f, tiles_n, v, n_tile);
   const TileRows where = rows.find(g.seg_off, v, small, s_owner);
   if constexpr (kSmall) {
     if (small) {
-      remainder_tile<T, BM, BN, MODE>(g, smem, where, n_tile);
+      remainder_tile<T, BM, BN, MODE>(g, smem, where, n_tile, narrow);
       return;
     }
   }
@@ -1453,7 +1496,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
 
   RowTiles<BM, kSmall, NW> rows;
   rows.scan(gd.seg_off, gd.n_expert, s_wave_sum);
-  const int live_d = rows.rows_f * tiles_n_d, live_s = rows.rows_s * tiles_n_d;
+  constexpr int kF = kSmall ? narrow_factor<BM, BN, GEMM_DGRAD>() : 1;
+  const bool narrow = kF > 1 && rows.rows_s * tiles_n_d <= kNarrowMax &&
+                      gd.out_feat >= kNarrowMinK;
+  const int cols_s = narrow ? tiles_n_d * kF : tiles_n_d;
+  const int live_d = rows.rows_f * tiles_n_d, live_s = rows.rows_s * cols_s;
   const int per_expert_w = tiles_n_w * tiles_m_w;
   const int live_w = per_expert_w * gw.n_expert;
   const int live = live_d + live_w + live_s;
@@ -1475,12 +1522,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
   }
   const bool small = t >= live_d;
   int v, n_tile;
-  if (small) tile_order(t - s_begin, rows.rows_s, tiles_n_d, v, n_tile);
+  if (small) tile_order(t - s_begin, rows.rows_s, cols_s, v, n_tile);
   else tile_order(t, rows.rows_f, tiles_n_d, v, n_tile);
   const TileRows where = rows.find(gd.seg_off, v, small, s_owner);
   if constexpr (kSmall) {
     if (small) {
-      remainder_tile<T, BM, BN, GEMM_DGRAD>(gd, smem, where, n_tile);
+      remainder_tile<T, BM, BN, GEMM_DGRAD>(gd, smem, where, n_tile, narrow);
       return;
     }
   }
@@ -1517,6 +1564,10 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
     // one remainder tile
     tiles_m = (int)(g.n_rows / BM) + g.n_expert;
     blocks = (int64_t)tiles_n * tiles_m;
+    // room for the narrow form of up to kNarrowMax remainder tiles
+    if (has_small_tiles<BM, BN, MODE>())
+      blocks += (int64_t)(narrow_factor<BM, BN, MODE>() - 1) *
+                std::min<int64_t>((int64_t)tiles_n * g.n_expert, kNarrowMax);
   }
   blocks = ceil_div(blocks, 8 * kXcdRun) * (8 * kXcdRun);  // whole runs for all 8 XCDs
   FMOE_REQUIRE(blocks < ((int64_t)1 << 31), FMOE_ERR_UNSUPPORTED,
@@ -1593,7 +1644,9 @@ static int launch_bwd_fused(const GemmArgs& gd, const GemmArgs& gw, hipStream_t 
   const int tiles_n_d = ceil_div(gd.in_feat, BN);
   const int tiles_n_w = ceil_div(gw.in_feat, BN), tiles_m_w = ceil_div(gw.out_feat, BM);
   int64_t blocks = (int64_t)tiles_n_d * (gd.n_rows / BM + (int64_t)gd.n_expert) +
-                   (int64_t)tiles_n_w * tiles_m_w * gw.n_expert;
+                   (int64_t)tiles_n_w * tiles_m_w * gw.n_expert +
+                   (int64_t)(narrow_factor<BM, BN, GEMM_DGRAD>() - 1) *
+                       std::min<int64_t>((int64_t)tiles_n_d * gd.n_expert, kNarrowMax);
   blocks = ceil_div(blocks, 8 * kXcdRun) * (8 * kXcdRun);
   FMOE_REQUIRE(blocks < ((int64_t)1 << 31), FMOE_ERR_UNSUPPORTED,
                "grouped GEMM: too many tiles");

@@ -93,6 +93,14 @@ def test_matrix_core_forced_tile(dt, tile, counts, in_f, out_f):
     _run(counts, in_f, out_f, DTYPES[dt], True, path=1 + tile, extra_rows=5)
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+def test_matrix_core_narrow_remainder_tiles(dt):
+    """With K >= 2048 and few remainder tiles in the launch, the remainders (1, 44, 64
+    and 100 rows here, behind 0 to 2 full tiles) run as 64-column (forward) and
+    128-column (dX) tiles; feature sizes that end inside such a tile, K with a tail."""
+    _run([300, 0, 257, 64, 1, 200, 513, 356], 2056, 2112, DTYPES[dt], True, path=0, extra_rows=3)
+
+
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 @pytest.mark.parametrize("with_bias", [True, False])
 @pytest.mark.parametrize("counts,in_f,out_f", SHAPES + FORCED)
