@@ -9,7 +9,9 @@
 //   place  one block per 2048 slots: per-wave LDS counters give every slot its
 //          rank among the earlier slots of the same expert    -> pos / inv / mask
 // No arrival-order atomics touch the result, so positions and drop masks are
-// the ones a sequential sweep over the slots would produce.
+// the ones a sequential sweep over the slots would produce.  Up to 4096 slots
+// and 512 experts fmoe_route runs the same three steps as ONE workgroup
+// (route_single_kernel): one launch instead of three.
 //
 // Semantics follow cuda/local_exchange.cuh:5-16,36-69 and
 // cuda/balancing.cuh:5-21,32-45 of the reference.
@@ -203,6 +205,116 @@ __global__ __launch_bounds__(kRouteThreads) void route_place_kernel(
   }
 }
 
+// ------------------------------------------------------------- single launch
+// The three steps above in ONE workgroup of 16 waves, for problems small enough
+// that three launches (and their gaps) cost more than the work: up to 4096 slots
+// and 512 experts (512 tokens, top-2: 22 -> 12 us per call; from 16384 slots on one
+// CU alone takes longer over the slots than three launches that use all of them:
+// 25 vs 19 us).  Wave w takes the w-th sixteenth of the 64-slot rows, so the
+// order of slots inside an expert is the ascending one of the three-kernel path
+// and the results are the same bit for bit.  A wave loads all its rows (at most
+// ROWS, kept in registers) in one go: with a load per loop trip the memory
+// latency of the dependent trips adds up.
+constexpr int kSingleThreads = 1024;
+constexpr int kSingleWaves = kSingleThreads / kWave;
+constexpr int kSingleMaxSlots = 4096;
+constexpr int kSingleRows = kSingleMaxSlots / kSingleThreads;   // 64-slot rows per wave
+constexpr int kSingleMaxExperts = 512;
+
+template <int ROWS>
+__global__ __launch_bounds__(kSingleThreads) void route_single_kernel(
+    const int64_t* __restrict__ gate, int64_t n, int n_expert, int64_t* __restrict__ count64,
+    int32_t* __restrict__ seg_off, int64_t* __restrict__ pos, int32_t* __restrict__ inv) {
+  extern __shared__ int32_t lds_single[];
+  int32_t* wave_cnt = lds_single;                            // [kSingleWaves][E]
+  int32_t* cnt = lds_single + kSingleWaves * n_expert;       // [E]
+  int32_t* off = cnt + n_expert;                             // [E+1]
+  const int w = threadIdx.x / kWave;
+  const int lane = lane_id();
+  for (int x = threadIdx.x; x < kSingleWaves * n_expert; x += kSingleThreads) wave_cnt[x] = 0;
+  __syncthreads();
+
+  const int rows = (int)((n + kWave - 1) / kWave);
+  const int rows_per_wave = (rows + kSingleWaves - 1) / kSingleWaves;
+  const int row_lo = w * rows_per_wave, row_hi = min(rows, row_lo + rows_per_wave);
+  int32_t keys[ROWS];
+#pragma unroll
+  for (int u = 0; u < ROWS; ++u) {
+    const int64_t i = (int64_t)(row_lo + u) * kWave + lane;
+    int32_t key = -1;
+    if (row_lo + u < row_hi && i < n) {
+      const int64_t g = gate[i];
+      if (g >= 0 && g < n_expert) key = (int32_t)g;
+    }
+    keys[u] = key;
+  }
+#pragma unroll
+  for (int u = 0; u < ROWS; ++u)
+    if (keys[u] >= 0) atomicAdd(&wave_cnt[w * n_expert + keys[u]], 1);
+  __syncthreads();
+  // per expert: its total, and where every wave's share starts inside its segment
+  for (int e = threadIdx.x; e < n_expert; e += kSingleThreads) {
+    int32_t run = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < kSingleWaves; ++w2) {
+      const int32_t t = wave_cnt[w2 * n_expert + e];
+      wave_cnt[w2 * n_expert + e] = run;
+      run += t;
+    }
+    cnt[e] = run;
+  }
+  __syncthreads();
+  if (threadIdx.x < kWave) {   // exclusive scan over the experts, 64 per step
+    int32_t carry = 0;
+    for (int base = 0; base < n_expert; base += kWave) {
+      const int e = base + lane;
+      const int32_t v = e < n_expert ? cnt[e] : 0;
+      int32_t incl = v;
+#pragma unroll
+      for (int d = 1; d < kWave; d <<= 1) {
+        const int32_t t = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += t;
+      }
+      if (e < n_expert) off[e] = carry + incl - v;
+      carry += __shfl(incl, kWave - 1, kWave);
+    }
+    if (lane == 0) off[n_expert] = carry;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n_expert; e += kSingleThreads) {
+    const int32_t o = off[e];
+#pragma unroll
+    for (int w2 = 0; w2 < kSingleWaves; ++w2) wave_cnt[w2 * n_expert + e] += o;
+    if (count64) count64[e] = cnt[e];
+    seg_off[e] = o;
+  }
+  if (threadIdx.x == 0) seg_off[n_expert] = off[n_expert];
+  __syncthreads();
+
+  const uint64_t lt_mask = ((uint64_t)1 << lane) - 1;
+  const int key_bits = 32 - __clz(max(n_expert - 1, 1));
+#pragma unroll
+  for (int u = 0; u < ROWS; ++u) {
+    if (row_lo + u >= row_hi) break;   // the same for the whole wave
+    const int64_t i = (int64_t)(row_lo + u) * kWave + lane;
+    const int32_t key = keys[u];
+    const bool valid = key >= 0;
+    uint64_t same = __ballot(valid);
+    for (int bit = 0; bit < key_bits; ++bit) {
+      const uint64_t vote = __ballot(valid && ((key >> bit) & 1));
+      same &= ((key >> bit) & 1) ? vote : ~vote;
+    }
+    const int rank = __popcll(same & lt_mask);
+    const bool first = valid && (same & lt_mask) == 0;
+    int32_t p = 0;
+    if (valid) p = wave_cnt[w * n_expert + key] + rank;
+    // every lane has read its counter before the leader of each expert advances it
+    if (valid && first) wave_cnt[w * n_expert + key] = p + __popcll(same);
+    if (valid) pos[p] = i;
+    if (inv != nullptr && i < n) inv[i] = valid ? p : -1;
+  }
+}
+
 // ------------------------------------------------------------------- limit
 // One thread per expert walks the workers in ascending order.
 __global__ __launch_bounds__(256) void limit_by_capacity_kernel(
@@ -320,10 +432,11 @@ extern "C" int64_t fmoe_route_workspace_bytes(int64_t numel, int32_t n_expert) {
   return route_ws_bytes(numel, n_expert);
 }
 
-extern "C" int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
-                          int64_t* count64, int32_t* seg_off, int64_t* pos,
-                          int32_t* inv, void* workspace, int64_t workspace_bytes,
-                          void* stream) {
+// `single_launch`: small problems may run as one workgroup without the workspace.
+static int route_impl(const int64_t* gate, int64_t numel, int32_t n_expert,
+                      int64_t* count64, int32_t* seg_off, int64_t* pos,
+                      int32_t* inv, void* workspace, int64_t workspace_bytes,
+                      void* stream, bool single_launch) {
   int rc = check_route_args(numel, n_expert);
   if (rc) return rc;
   FMOE_REQUIRE(seg_off != nullptr, FMOE_ERR_INVALID, "route: seg_off is null");
@@ -333,6 +446,13 @@ extern "C" int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
   rc = carve_ws(workspace, workspace_bytes, numel, n_expert, &ws);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
+  if (single_launch && numel <= kSingleMaxSlots && n_expert <= kSingleMaxExperts) {
+    const size_t lds = ((kSingleWaves + 2) * n_expert + 1) * sizeof(int32_t);
+    hipLaunchKernelGGL(route_single_kernel<kSingleRows>, dim3(1), dim3(kSingleThreads), lds, s,
+                       gate, numel, (int)n_expert, count64, seg_off, pos, inv);
+    FMOE_LAUNCH_CHECK("route_single");
+    return FMOE_OK;
+  }
   if (ws.n_blocks > 0) {
     hipLaunchKernelGGL(route_hist_kernel, dim3(ws.n_blocks), dim3(kRouteThreads),
                        n_expert * sizeof(int32_t), s, gate, numel, (int)n_expert,
@@ -355,6 +475,14 @@ extern "C" int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
   return FMOE_OK;
 }
 
+extern "C" int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
+                          int64_t* count64, int32_t* seg_off, int64_t* pos,
+                          int32_t* inv, void* workspace, int64_t workspace_bytes,
+                          void* stream) {
+  return route_impl(gate, numel, n_expert, count64, seg_off, pos, inv, workspace,
+                    workspace_bytes, stream, true);
+}
+
 extern "C" int fmoe_route_static(const int64_t* gate, int64_t numel, int32_t n_expert,
                                  int64_t* count64, int32_t* seg_off, int64_t* pos,
                                  int32_t* inv, void* stream) {
@@ -370,8 +498,9 @@ extern "C" int fmoe_route_static(const int64_t* gate, int64_t numel, int32_t n_e
   if (rc) return rc;
   // every block of the histogram kernel overwrites its whole row of the table
   // before anything reads it, so what the last call left behind needs no clearing
-  return fmoe_route(gate, numel, n_expert, count64, seg_off, pos, inv, ws, kStaticScratchBytes,
-                    stream);
+  // (always the three-kernel form: it is the one that uses the scratch buffer)
+  return route_impl(gate, numel, n_expert, count64, seg_off, pos, inv, ws, kStaticScratchBytes,
+                    stream, false);
 }
 
 extern "C" int fmoe_assign_pos(int32_t* cum_count, const int64_t* gate,

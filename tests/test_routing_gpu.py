@@ -28,6 +28,11 @@ CASES = [  # n_tokens, top_k, n_expert, drop
     (8192, 8, 128, 0.0),     # config 5 shape
     (5000, 2, 1000, 0.2),    # many experts
     (3000, 2, 4096, 0.0),    # the LDS limit
+    (4096, 1, 512, 0.05),    # the largest problem routed by a single workgroup
+    (4097, 1, 512, 0.05),    # one slot more: three kernels
+    (1363, 3, 7, 0.05),      # 4089 slots: ragged last row
+    (40000, 2, 64, 0.1),     # 80000 slots: three kernels
+    (1500, 2, 513, 0.0),     # one expert too many for the single workgroup
 ]
 
 
