@@ -35,6 +35,7 @@ SHAPES = [  # rows per expert, in_feat, out_feat
     ([7, 250], 136, 72),                          # widths that are no multiple of a tile
     ([0, 0, 0], 64, 64),                          # no rows at all
     ([700], 1024, 64),
+    ([300, 0, 129, 64, 1, 0, 513, 356], 264, 2048),   # K = 2048: narrow remainder tiles of dX
 ]
 
 
