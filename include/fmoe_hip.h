@@ -98,14 +98,17 @@ int fmoe_assign_pos(int32_t* cum_count, const int64_t* gate, int64_t* pos,
  *   inv         (optional, int32[numel])
  * Stands in for fmoe.functions.count_by_gate + prepare_forward
  * (fmoe/functions.py:28-75) without their five device-to-host copies.
+ * Three launches (histogram, scans, placement); up to 4096 slots and 512
+ * experts one workgroup does all three in a single launch, same results.  The
+ * workspace is required either way.
  */
 int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
                int64_t* count64, int32_t* seg_off, int64_t* pos, int32_t* inv,
                void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
- * fmoe_route for callers that cannot allocate: the same kernels and results,
- * with the per-block histograms in a buffer built into the library
+ * fmoe_route for callers that cannot allocate: the three-launch kernels and
+ * the same results, with the per-block histograms in a buffer built into the library
  * (FMOE_ROUTE_STATIC_SCRATCH_BYTES per GPU, held until the process ends) instead
  * of a workspace argument.  It calls no allocating routine, so it may be used
  * under HIP graph capture, in serving loops and in harnesses that forbid
