@@ -284,6 +284,42 @@ def test_dropped_slots_flow_through_the_layer():
     assert max_rel_err(out, want) <= 1e-4
 
 
+@pytest.mark.parametrize("n_expert,top_k", [(24, 20), (80, 70)])
+def test_top_k_beyond_the_gate_and_combine_kernels(n_expert, top_k):
+    """top_k above 16 leaves the fused gate kernel for torch.topk + softmax (the
+    reference's own formulation, naive_gate.py:31-38); above 64 the layer also
+    leaves the fused combine kernels for the reference-shaped route (MOEScatter ->
+    experts -> MOEGather + bmm).  Both against the brute force, with gradients."""
+    from fastmoe_amd import FMoETransformerMLP
+
+    torch.manual_seed(21)
+    moe = FMoETransformerMLP(n_expert, 32, 48, top_k=top_k).cuda()
+    x = torch.randn(150, 32)
+    dy = torch.randn(150, 32)
+    x_dev = x.cuda().requires_grad_(True)
+    out = moe(x_dev)
+    out.backward(dy.cuda())
+    with torch.no_grad():
+        idx, score = moe.gate(x.cuda())
+    assert tuple(idx.shape) == (150, top_k)
+    assert all(len(set(r)) == top_k for r in idx.cpu().tolist())     # k distinct experts
+    ex = moe.experts
+    ps = [p.detach().double().cpu().requires_grad_(True)
+          for p in (ex.htoh4.weight, ex.htoh4.bias, ex.h4toh.weight, ex.h4toh.bias)]
+    xr = x.double().requires_grad_(True)
+    # the gate itself, recomputed on the host: logits -> top-k -> softmax over the k values
+    logits = xr @ moe.gate.gate.weight.detach().double().cpu().t() \
+        + moe.gate.gate.bias.detach().double().cpu()
+    ref_score = torch.softmax(torch.gather(logits, 1, idx.cpu()), dim=-1)
+    assert (ref_score - score.double().cpu()).abs().max().item() <= 1e-5
+    want = O.brute_force_moe_mlp(xr, idx.cpu(), ref_score, *ps)
+    want.backward(dy.double())
+    assert max_rel_err(out, want) <= 1e-4
+    assert max_rel_err(x_dev.grad, xr.grad) <= 1e-4
+    for dev, ref in zip((ex.htoh4.weight, ex.htoh4.bias, ex.h4toh.weight, ex.h4toh.bias), ps):
+        assert max_rel_err(dev.grad, ref.grad) <= 1e-4
+
+
 def test_config2_full_size_layer_against_brute_force():
     """The benchmark workload itself (8192 tokens, d_model 1024, d_hidden 4096,
     16 experts, top-2, bf16): output, input gradient and all four expert
