@@ -1060,13 +1060,17 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   const bool fuse_act = MODE == GEMM_DGRAD && g.act_pre != nullptr;
   static_assert(BM * kLdc * 2 <= kActTabLdsOffset, "the table sits behind the largest staged tile");
   float* act_tab = reinterpret_cast<float*>(smem + kActTabLdsOffset / 2);
-  constexpr int kTabPerThread = (kActTabCount / 4 + NT - 1) / NT;
-  uint4 tab_regs[kTabPerThread];
-  if (MODE == GEMM_DGRAD && fuse_act) {
-    const uint4* src = reinterpret_cast<const uint4*>(g.act_table + kActTabFirst);
+  // (an even split: a guarded load into the array would put it into scratch
+  // memory, one load and one wait at a time)
+  static_assert((kActTabCount / 4) % NT == 0, "the table splits evenly over the threads");
+  constexpr int kTabPerThread = kActTabCount / 4 / NT;
+  i32x4_t tab_regs[kTabPerThread];
 #pragma unroll
-    for (int i = 0; i < kTabPerThread; ++i)
-      if (tid + i * NT < kActTabCount / 4) tab_regs[i] = src[tid + i * NT];
+  for (int i = 0; i < kTabPerThread; ++i) tab_regs[i] = i32x4_t{0, 0, 0, 0};
+  if (MODE == GEMM_DGRAD && fuse_act) {
+    const i32x4_t* src = reinterpret_cast<const i32x4_t*>(g.act_table + kActTabFirst);
+#pragma unroll
+    for (int i = 0; i < kTabPerThread; ++i) tab_regs[i] = src[tid + i * NT];
   }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -1093,7 +1097,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   if (MODE == GEMM_DGRAD && fuse_act) {
 #pragma unroll
     for (int i = 0; i < kTabPerThread; ++i)
-      if (tid + i * NT < kActTabCount / 4) reinterpret_cast<uint4*>(act_tab)[tid + i * NT] = tab_regs[i];
+      reinterpret_cast<i32x4_t*>(act_tab)[tid + i * NT] = tab_regs[i];
   }
   __syncthreads();
   // every thread moves one fixed 16-byte column pack of every kRowsPerStep-th row
