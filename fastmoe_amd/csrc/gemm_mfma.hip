@@ -689,22 +689,32 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   struct alignas(8) Out4 { T v[4]; };
   constexpr int kLdc = BN + 8;   // elements per staged row
   T* stage_c = reinterpret_cast<T*>(smem);
+  // (only the forward product has a bias; elsewhere the sums are rounded as they
+  // are: adding a zero would cost an instruction per value, which the compiler may
+  // not drop because of -0.  ONE code path: two variants of this loop made the
+  // register allocator shuffle the accumulators inside the K loop.)
+  {
+    constexpr bool kBias = MODE == GEMM_FWD;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int col = wave_n * (BN / WN) + j * 16 + 4 * (lane >> 4);
-    float bv[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias && n0 + col < N) {
-      const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
+    for (int j = 0; j < TN; ++j) {
+      const int col = wave_n * (BN / WN) + j * 16 + 4 * (lane >> 4);
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (kBias) {
+        if (bias && n0 + col < N) {
+          const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
 #pragma unroll
-      for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
-    }
+          for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
+        }
+      }
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int row = wave_m * (BM / WM) + i * 16 + (lane & 15);
-      Out4 o;
+      for (int i = 0; i < TM; ++i) {
+        const int row = wave_m * (BM / WM) + i * 16 + (lane & 15);
+        Out4 o;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) o.v[c] = Elem<T>::from_acc(acc[i][j][c] + bv[c]);
-      *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
+        for (int c = 0; c < 4; ++c)
+          o.v[c] = Elem<T>::from_acc(kBias ? acc[i][j][c] + bv[c] : acc[i][j][c]);
+        *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
+      }
     }
   }
   __syncthreads();
@@ -1072,25 +1082,34 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
 #pragma unroll
     for (int i = 0; i < kTabPerThread; ++i) tab_regs[i] = src[tid + i * NT];
   }
+  // (only the forward product has a bias; elsewhere the sums are rounded as they
+  // are: adding a zero would cost an instruction per value, which the compiler may
+  // not drop because of -0.  ONE code path: two variants of this loop made the
+  // register allocator shuffle the accumulators inside the K loop.)
+  {
+    constexpr bool kBias = MODE == GEMM_FWD;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
+    for (int j = 0; j < TN; ++j) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int col = wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (bias && n0 + col < N) {
-        const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
+      for (int q = 0; q < 4; ++q) {
+        const int col = wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (kBias) {
+          if (bias && n0 + col < N) {
+            const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
-      }
+            for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
+          }
+        }
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row = wave_m * (BM / WM) + i * 32 + (lane & 31);
-        Out4 o;
+        for (int i = 0; i < TM; ++i) {
+          const int row = wave_m * (BM / WM) + i * 32 + (lane & 31);
+          Out4 o;
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-          o.v[c] = Elem<T>::from_acc(acc[i][j][4 * q + c] + bv[c]);
-        *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
+          for (int c = 0; c < 4; ++c)
+            o.v[c] = Elem<T>::from_acc(kBias ? acc[i][j][4 * q + c] + bv[c] : acc[i][j][4 * q + c]);
+          *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
+        }
       }
     }
   }
@@ -1312,6 +1331,21 @@ __device__ __forceinline__ int tile_number(int pid, int live) {
   return (slot / run) * (8 * run) + (pid & 7) * run + slot % run;
 }
 
+// Inclusive prefix sum over the 64 lanes of a wave with data-parallel-primitive
+// moves (no trips through the LDS crossbar: every workgroup runs this before its
+// first copy): shifts by 1, 2, 4, 8 inside each row of 16 lanes, then lane 15 of
+// rows 0 and 2 added to rows 1 and 3, then lane 31 added to rows 2 and 3.  A lane
+// without a source, or outside the row mask, adds the 0 passed as the old value.
+__device__ __forceinline__ int wave_inclusive_sum(int x) {
+  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false);  // row_shr:1
+  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false);  // row_shr:2
+  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false);  // row_shr:4
+  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false);  // row_shr:8
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false);  // row_bcast:15
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false);  // row_bcast:31
+  return x;
+}
+
 // Row tiles of a ragged product.  The BM-row tiles of all experts are numbered
 // first, one expert after the other, the remainder tiles behind them.
 //
@@ -1355,16 +1389,9 @@ struct RowTiles {
         mine_s += sm;
       }
     }
-    int incl_f = mine_f, incl_s = mine_s;  // inclusive scans inside the wave
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int up_f = __shfl_up(incl_f, d, 64);
-      if (lane >= d) incl_f += up_f;
-      if (SMALL) {
-        const int up_s = __shfl_up(incl_s, d, 64);
-        if (lane >= d) incl_s += up_s;
-      }
-    }
+    // inclusive scans inside the wave
+    const int incl_f = wave_inclusive_sum(mine_f);
+    const int incl_s = SMALL ? wave_inclusive_sum(mine_s) : 0;
     first_f = incl_f - mine_f;
     first_s = incl_s - mine_s;
     if (by_lane) {
