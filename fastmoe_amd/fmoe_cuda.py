@@ -555,6 +555,28 @@ def set_gemm_path(path: int) -> None:
     _lib.check(_L.fmoe_set_gemm_path(path), "set_gemm_path")
 
 
+def _hooked(name, fn):
+    """A compiled operator that reports to `profile_hook` the way the ctypes ones do."""
+
+    def op(*args, **kwargs):
+        if profile_hook is None or (profile_only is not None and name not in profile_only):
+            return fn(*args, **kwargs)
+        first = next((a for a in args if isinstance(a, torch.Tensor) and a.is_cuda), None)
+        if first is None:
+            return fn(*args, **kwargs)
+        stream = torch.cuda.current_stream(first.device)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        out = fn(*args, **kwargs)
+        end.record(stream)
+        profile_hook(name, start, end)
+        return out
+
+    op.__name__ = name
+    op.__doc__ = fn.__doc__
+    return op
+
+
 BINDING = "ctypes"
 if os.environ.get("FMOE_BINDING", "ctypes").lower() in ("compiled", "ext", "pybind"):
     from . import _ext
@@ -566,5 +588,5 @@ if os.environ.get("FMOE_BINDING", "ctypes").lower() in ("compiled", "ext", "pybi
                   "grouped_linear_bwd", "gather_combine_fwd", "gather_combine_bwd",
                   "scatter_reduce", "topk_softmax_fwd", "topk_softmax_bwd", "gelu_fwd", "gelu_bwd",
                   "set_gemm_path", "_seg_off_from_counts"):
-        globals()[_name] = getattr(_compiled, _name)
+        globals()[_name] = _hooked(_name, getattr(_compiled, _name))
     BINDING = "compiled"
