@@ -693,31 +693,32 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   // are: adding a zero would cost an instruction per value, which the compiler may
   // not drop because of -0.  ONE code path: two variants of this loop made the
   // register allocator shuffle the accumulators inside the K loop.)
-  {
-    constexpr bool kBias = MODE == GEMM_FWD;
+  constexpr bool kBias = MODE == GEMM_FWD;
+  float bv[TN][4];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+  for (int j = 0; j < TN; ++j) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) bv[j][c] = 0.f;
+    if constexpr (kBias) {
       const int col = wave_n * (BN / WN) + j * 16 + 4 * (lane >> 4);
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if constexpr (kBias) {
-        if (bias && n0 + col < N) {
-          const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
+      if (bias && n0 + col < N) {
+        const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
 #pragma unroll
-          for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row = wave_m * (BM / WM) + i * 16 + (lane & 15);
-        Out4 o;
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-          o.v[c] = Elem<T>::from_acc(kBias ? acc[i][j][c] + bv[c] : acc[i][j][c]);
-        *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
+        for (int c = 0; c < 4; ++c) bv[j][c] = Elem<T>::to_acc(b4.v[c]);
       }
     }
   }
-  __syncthreads();
+  // block (i, j) of the wave's accumulators, rounded, into the staged tile
+  auto stage_block = [&](auto i_tag, auto j_tag) {
+    constexpr int i = decltype(i_tag)::value, j = decltype(j_tag)::value;
+    const int col = wave_n * (BN / WN) + j * 16 + 4 * (lane >> 4);
+    const int row = wave_m * (BM / WM) + i * 16 + (lane & 15);
+    Out4 o;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      o.v[c] = Elem<T>::from_acc(kBias ? acc[i][j][c] + bv[j][c] : acc[i][j][c]);
+    *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
+  };
   // every thread moves one fixed 16-byte column pack of every kRowsPerStep-th row
   constexpr int kRowPacks = BN / 8;                  // 16-byte packs per tile row
   constexpr int kRowsPerStep = NT / kRowPacks;
@@ -728,15 +729,62 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   const T* sp = stage_c + r0 * kLdc + pk * 8;
   // Rows past the expert's last one are cut off by the buffer descriptor (the
   // bytes of this tile end with the last valid row), so the loop carries no
-  // per-row condition.
+  // per-row condition; a pack past the last column (N is a multiple of 8: a pack
+  // is all in or all out) gets an offset no descriptor reaches.
   const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(C + (int64_t)m0 * ldc + n0), (short)0, ((m_valid - 1) * ldc + n_valid) * 2,
       kRsrcFlags);
-  const int c_off = (r0 * ldc + pk * 8) * 2;
-  if (n0 + pk * 8 < N) {  // N is a multiple of 8: a pack is all in or all out
+  const int c_off = n0 + pk * 8 < N ? (r0 * ldc + pk * 8) * 2 : (int)kOutOfRange;
+  // The upper half of every wave's rows is staged while the packs of the lower
+  // half are on their way out: the stores leave at the address unit's pace (about
+  // 30 cycles per wave instruction), the staging is conversion work for the vector
+  // unit, and a wave that issued them back to back would sit at the stores.
+  constexpr int kBand = BM / WM / kRowsPerStep;      // store steps per band of wave rows
+  constexpr bool kOverlap = TM % 2 == 0 && (BM / WM) % (2 * kRowsPerStep) == 0;
+  if constexpr (kOverlap) {
+    constexpr int kHalf = kSteps / 2, kBlocks = TM / 2 * TN;
+    // store step of the s-th pack of half h
+    auto step_of = [](int h, int s2) constexpr {
+      return s2 / (kBand / 2) * kBand + h * (kBand / 2) + s2 % (kBand / 2);
+    };
+    static_for<kBlocks>([&](auto b_tag) {
+      constexpr int b = decltype(b_tag)::value;
+      stage_block(std::integral_constant<int, b % (TM / 2)>{}, std::integral_constant<int, b / (TM / 2)>{});
+    });
+    __syncthreads();
     // Every pack gets registers of its own: a store holds its data registers
     // until memory has acknowledged it, so a register reused for a later pack
     // would make that pack wait for a full store round trip.
+    i32x4_t v[kSteps];
+#pragma unroll
+    for (int s2 = 0; s2 < kHalf; ++s2)
+      v[s2] = *reinterpret_cast<const i32x4_t*>(sp + step_of(0, s2) * kRowsPerStep * kLdc);
+    static_for<kHalf>([&](auto s_tag) {
+      constexpr int s2 = decltype(s_tag)::value;
+      __builtin_amdgcn_raw_buffer_store_b128(
+          v[s2], c_rsrc, c_off + step_of(0, s2) * kRowsPerStep * ldc * 2, 0, 0);
+      constexpr int b_lo = s2 * kBlocks / kHalf, b_hi = (s2 + 1) * kBlocks / kHalf;
+      static_for<b_hi - b_lo>([&](auto d_tag) {
+        constexpr int b = b_lo + decltype(d_tag)::value;
+        stage_block(std::integral_constant<int, TM / 2 + b % (TM / 2)>{},
+                    std::integral_constant<int, b / (TM / 2)>{});
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __syncthreads();
+#pragma unroll
+    for (int s2 = 0; s2 < kHalf; ++s2)
+      v[kHalf + s2] = *reinterpret_cast<const i32x4_t*>(sp + step_of(1, s2) * kRowsPerStep * kLdc);
+#pragma unroll
+    for (int s2 = 0; s2 < kHalf; ++s2)
+      __builtin_amdgcn_raw_buffer_store_b128(
+          v[kHalf + s2], c_rsrc, c_off + step_of(1, s2) * kRowsPerStep * ldc * 2, 0, 0);
+  } else {
+    static_for<TM * TN>([&](auto b_tag) {
+      constexpr int b = decltype(b_tag)::value;
+      stage_block(std::integral_constant<int, b % TM>{}, std::integral_constant<int, b / TM>{});
+    });
+    __syncthreads();
     i32x4_t v[kSteps];
 #pragma unroll
     for (int u = 0; u < kSteps; ++u)
@@ -747,6 +795,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
                                              0);
   }
 }
+
 
 // gemm_tile() with 32x32x16 MFMAs (the wave's patch as a grid of 32x32
 // accumulators): used for DGRAD and WGRAD.
@@ -1084,41 +1133,39 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   }
   // (only the forward product has a bias; elsewhere the sums are rounded as they
   // are: adding a zero would cost an instruction per value, which the compiler may
-  // not drop because of -0.  ONE code path: two variants of this loop made the
-  // register allocator shuffle the accumulators inside the K loop.)
-  {
-    constexpr bool kBias = MODE == GEMM_FWD;
+  // not drop because of -0)
+  constexpr bool kBias = MODE == GEMM_FWD;
+  // 4 columns of block (i, j), column group q, rounded, into the staged tile
+  auto stage_block = [&](auto i_tag, auto j_tag, auto q_tag) {
+    constexpr int i = decltype(i_tag)::value, j = decltype(j_tag)::value;
+    constexpr int q = decltype(q_tag)::value;
+    const int col = wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
+    const int row = wave_m * (BM / WM) + i * 32 + (lane & 31);
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (kBias) {
+      if (bias && n0 + col < N) {
+        const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int col = wave_n * (BN / WN) + j * 32 + 8 * q + 4 * (lane >> 5);
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (kBias) {
-          if (bias && n0 + col < N) {
-            const Out4 b4 = *reinterpret_cast<const Out4*>(bias + n0 + col);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const int row = wave_m * (BM / WM) + i * 32 + (lane & 31);
-          Out4 o;
-#pragma unroll
-          for (int c = 0; c < 4; ++c)
-            o.v[c] = Elem<T>::from_acc(kBias ? acc[i][j][4 * q + c] + bv[c] : acc[i][j][4 * q + c]);
-          *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
-        }
+        for (int c = 0; c < 4; ++c) bv[c] = Elem<T>::to_acc(b4.v[c]);
       }
     }
-  }
-  if (MODE == GEMM_DGRAD && fuse_act) {
+    Out4 o;
 #pragma unroll
-    for (int i = 0; i < kTabPerThread; ++i)
-      reinterpret_cast<i32x4_t*>(act_tab)[tid + i * NT] = tab_regs[i];
-  }
-  __syncthreads();
+    for (int c = 0; c < 4; ++c)
+      o.v[c] = Elem<T>::from_acc(kBias ? acc[i][j][4 * q + c] + bv[c] : acc[i][j][4 * q + c]);
+    *reinterpret_cast<Out4*>(stage_c + row * kLdc + col) = o;
+  };
+  // blocks [lo, hi) of the wave in the order (j, q, i): i runs over rows [i_lo, i_lo + n_i)
+  auto stage_blocks = [&](auto ilo_tag, auto ni_tag, auto lo_tag, auto hi_tag) {
+    constexpr int i_lo = decltype(ilo_tag)::value, n_i = decltype(ni_tag)::value;
+    constexpr int lo = decltype(lo_tag)::value, hi = decltype(hi_tag)::value;
+    static_for<hi - lo>([&](auto d_tag) {
+      constexpr int b = lo + decltype(d_tag)::value;
+      stage_block(std::integral_constant<int, i_lo + b % n_i>{},
+                  std::integral_constant<int, b / n_i / 4>{},
+                  std::integral_constant<int, b / n_i % 4>{});
+    });
+  };
   // every thread moves one fixed 16-byte column pack of every kRowsPerStep-th row
   constexpr int kRowPacks = BN / 8;                  // 16-byte packs per tile row
   constexpr int kRowsPerStep = NT / kRowPacks;
@@ -1134,6 +1181,61 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
       (void*)(C + (int64_t)m0 * ldc + n0), (short)0, ((m_valid - 1) * ldc + n_valid) * 2,
       kRsrcFlags);
   const int c_off = (r0 * ldc + pk * 8) * 2;
+  // The upper half of every wave's rows is staged while the packs of the lower
+  // half are on their way out (see gemm_tile16); with the activation's backward
+  // fused in, the whole tile is staged first.
+  constexpr int kBand = BM / WM / kRowsPerStep;      // store steps per band of wave rows
+  constexpr bool kOverlap = TM % 2 == 0 && (BM / WM) % (2 * kRowsPerStep) == 0;
+  constexpr int kHalfRows = kOverlap ? TM / 2 : TM;  // row blocks staged before the first barrier
+  constexpr int kBlocksLo = kHalfRows * TN * 4, kBlocksHi = (TM - kHalfRows) * TN * 4;
+  stage_blocks(std::integral_constant<int, 0>{}, std::integral_constant<int, kHalfRows>{},
+               std::integral_constant<int, 0>{}, std::integral_constant<int, kBlocksLo>{});
+  if (MODE == GEMM_DGRAD && fuse_act) {
+#pragma unroll
+    for (int i = 0; i < kTabPerThread; ++i)
+      reinterpret_cast<i32x4_t*>(act_tab)[tid + i * NT] = tab_regs[i];
+  }
+  if constexpr (kOverlap) {
+    if (!(MODE == GEMM_DGRAD && fuse_act)) {
+      constexpr int kHalf = kSteps / 2;
+      // store step of the s-th pack of half h
+      auto step_of = [](int h, int s2) constexpr {
+        return s2 / (kBand / 2) * kBand + h * (kBand / 2) + s2 % (kBand / 2);
+      };
+      const int c_off_v = n0 + pk * 8 < N ? c_off : (int)kOutOfRange;  // N is a multiple of 8
+      __syncthreads();
+      // Every pack gets registers of its own: a store holds its data registers
+      // until memory has acknowledged it.
+      i32x4_t v[kSteps];
+#pragma unroll
+      for (int s2 = 0; s2 < kHalf; ++s2)
+        v[s2] = *reinterpret_cast<const i32x4_t*>(sp + step_of(0, s2) * kRowsPerStep * kLdc);
+      static_for<kHalf>([&](auto s_tag) {
+        constexpr int s2 = decltype(s_tag)::value;
+        __builtin_amdgcn_raw_buffer_store_b128(
+            v[s2], c_rsrc, c_off_v + step_of(0, s2) * kRowsPerStep * ldc * 2, 0, 0);
+        stage_blocks(std::integral_constant<int, kHalfRows>{},
+                     std::integral_constant<int, TM - kHalfRows>{},
+                     std::integral_constant<int, s2 * kBlocksHi / kHalf>{},
+                     std::integral_constant<int, (s2 + 1) * kBlocksHi / kHalf>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      __syncthreads();
+#pragma unroll
+      for (int s2 = 0; s2 < kHalf; ++s2)
+        v[kHalf + s2] =
+            *reinterpret_cast<const i32x4_t*>(sp + step_of(1, s2) * kRowsPerStep * kLdc);
+#pragma unroll
+      for (int s2 = 0; s2 < kHalf; ++s2)
+        __builtin_amdgcn_raw_buffer_store_b128(
+            v[kHalf + s2], c_rsrc, c_off_v + step_of(1, s2) * kRowsPerStep * ldc * 2, 0, 0);
+      return;
+    }
+    stage_blocks(std::integral_constant<int, kHalfRows>{},
+                 std::integral_constant<int, TM - kHalfRows>{}, std::integral_constant<int, 0>{},
+                 std::integral_constant<int, kBlocksHi>{});
+  }
+  __syncthreads();
   if (MODE == GEMM_DGRAD && fuse_act) {
     // dx = dH * gelu'(pre): the staged dH (already rounded to the storage type,
     // as a separate activation kernel would read it) times the table value of
