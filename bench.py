@@ -184,6 +184,7 @@ def kernel_work(cfg: dict, n_valid: int):
     gemm = 2.0 * n_valid * d * h
     return {
         "grouped_linear_fwd": ("flop", gemm),
+        "grouped_linear_fwd_act": ("flop", gemm),        # first layer, gelu from the same tiles
         "grouped_linear_dgrad": ("flop", gemm),
         "grouped_linear_wgrad": ("flop", gemm),
         "grouped_linear_bwd": ("flop", 2.0 * gemm),      # dX and dW in one launch

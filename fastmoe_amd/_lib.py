@@ -45,6 +45,9 @@ SIGNATURES = {
     "fmoe_grouped_linear_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_int64, c_int64, c_int64,
                                         c_int64, c_int, c_void_p]),
+    "fmoe_grouped_linear_fwd_act": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                            c_int64, c_int, c_void_p]),
     "fmoe_grouped_linear_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p, c_int64,
                                         c_int64, c_int64, c_int64, c_int, c_void_p]),

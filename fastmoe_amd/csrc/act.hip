@@ -256,6 +256,18 @@ int gelu_bwd_table(int dtype, hipStream_t s, const float** table) {
   return FMOE_OK;
 }
 
+// Device address of the gelu(x) table of a 16-bit dtype (65536 results, indexed
+// by the bit pattern of x), built on first use.
+int gelu_fwd_table(int dtype, hipStream_t s, const uint16_t** table) {
+  int cus = 0;
+  const int rc = ensure_tables(s, &cus);
+  if (rc) return rc;
+  uint16_t* base = nullptr;
+  FMOE_HIP_CHECK(hipGetSymbolAddress((void**)&base, HIP_SYMBOL(g_gelu_fwd_tab)));
+  *table = base + (dtype == FMOE_BF16 ? 0 : kTabFwd);
+  return FMOE_OK;
+}
+
 }  // namespace fmoe
 
 using namespace fmoe;

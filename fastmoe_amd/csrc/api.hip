@@ -13,6 +13,9 @@ static int g_gemm_path = 0;  // 0 = automatic, 1 = scalar kernel only (2..5 set 
 // tuning aid: FMOE_GEMM_TILE=1..4 forces one MFMA tile configuration (0 / unset = automatic)
 static const int g_env_tile = getenv("FMOE_GEMM_TILE") ? atoi(getenv("FMOE_GEMM_TILE")) : 0;
 static int g_tile = g_env_tile;
+// tuning aid: FMOE_FUSE_FWD_ACT=0 keeps the forward activation a kernel of its own
+static const bool g_fuse_fwd_act =
+    !(getenv("FMOE_FUSE_FWD_ACT") && atoi(getenv("FMOE_FUSE_FWD_ACT")) == 0);
 
 int set_error(int code, const char* fmt, ...) {
   va_list ap;
@@ -187,6 +190,38 @@ extern "C" int fmoe_grouped_linear_fwd(const void* x, const void* w,
                "grouped_linear_fwd: null pointer");
   GemmArgs g{x, w, y, bias, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
   return run_gemm(GEMM_FWD, g, dtype, (hipStream_t)stream);
+}
+
+// Forward of the grouped linear layer with the activation behind it: y as
+// fmoe_grouped_linear_fwd writes it and y_act = gelu(y), from the same tiles where
+// the bf16 matrix-core kernel runs, by the activation kernel over y otherwise.
+extern "C" int fmoe_grouped_linear_fwd_act(const void* x, const void* w, const void* bias,
+                                           const int32_t* seg_off, void* y, void* y_act,
+                                           int64_t n_rows, int64_t in_feat, int64_t out_feat,
+                                           int64_t n_expert, int dtype, void* stream) {
+  int rc = check_linear("grouped_linear_fwd_act", n_rows, in_feat, out_feat, n_expert, dtype);
+  if (rc) return rc;
+  if (n_rows == 0) return FMOE_OK;
+  FMOE_REQUIRE(x && w && seg_off && y && y_act, FMOE_ERR_INVALID,
+               "grouped_linear_fwd_act: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  GemmArgs g{x, w, y, bias, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
+  // Worth it from about 768 rows per expert on (measured: 12 % of GEMM + activation
+  // kernel at 1024 rows per expert, 5 % at 4096, level at 512, where half of the tiles
+  // are remainder tiles that pay the table and the second store for few rows); a
+  // forced tile shape (tests, tuning) takes the fused tiles at any size.
+  const bool fused = dtype == FMOE_BF16 && g_gemm_path == 0 && (uintptr_t)y_act % 16 == 0 &&
+                     g_fuse_fwd_act && (g_tile != 0 || n_rows >= 768 * n_expert) &&
+                     gemm_mfma_supported(GEMM_FWD, g, dtype);
+  if (fused) {
+    rc = gelu_fwd_table(dtype, s, &g.act_fwd_table);
+    if (rc) return rc;
+    g.act_out = y_act;
+    return launch_gemm_mfma(GEMM_FWD, g, dtype, s);
+  }
+  rc = run_gemm(GEMM_FWD, g, dtype, s);
+  if (rc) return rc;
+  return fmoe_gelu_fwd(y, y_act, n_rows * out_feat, seg_off + n_expert, out_feat, dtype, stream);
 }
 
 // Backward of the grouped linear layer; with act_pre, dx is further multiplied

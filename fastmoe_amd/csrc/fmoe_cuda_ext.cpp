@@ -125,6 +125,31 @@ Tensor grouped_linear_fwd(Tensor x, Tensor seg_off, Tensor weight, OptTensor bia
   return y;
 }
 
+// grouped_linear_fwd(..., with_gelu): y, or (y, gelu(y)) from the same launch
+py::object grouped_linear_fwd_any(Tensor x, Tensor seg_off, Tensor weight, OptTensor bias,
+                                  bool with_gelu) {
+  if (!with_gelu) return py::cast(grouped_linear_fwd(x, seg_off, weight, bias));
+  dev(x, "x");
+  dev(weight, "weight", x.scalar_type());
+  dev(seg_off, "seg_off", at::kInt);
+  need(x.dim() == 2 && weight.dim() == 3, "x must be 2-d and weight 3-d");
+  const int64_t e = weight.size(0), out_f = weight.size(1), in_f = weight.size(2);
+  need(x.size(1) == in_f, "x and weight disagree on the input features");
+  need(seg_off.numel() == e + 1, "seg_off must have E+1 entries");
+  if (bias.has_value() && bias->defined()) {
+    dev(*bias, "bias", x.scalar_type());
+    need(bias->dim() == 2 && bias->size(0) == e && bias->size(1) == out_f, "bias must be [E, out]");
+  }
+  c10::DeviceGuard guard(x.device());
+  Tensor y = torch::empty({x.size(0), out_f}, x.options());
+  Tensor y_act = torch::empty_like(y);
+  check(fmoe_grouped_linear_fwd_act(x.data_ptr(), weight.data_ptr(), ptr(bias),
+                                    seg_off.data_ptr<int32_t>(), y.data_ptr(), y_act.data_ptr(),
+                                    x.size(0), in_f, out_f, e, dt(x, "x"), stream_of(x)),
+        "grouped_linear_fwd_act");
+  return py::make_tuple(y, y_act);
+}
+
 std::tuple<OptTensor, OptTensor, OptTensor> grouped_linear_bwd(Tensor dy, Tensor x, Tensor seg_off,
                                                                Tensor weight, bool need_bias,
                                                                bool need_dx, bool need_dw,
@@ -412,8 +437,8 @@ PYBIND11_MODULE(fmoe_cuda, m) {
   m.def("route", &route, py::arg("gate"), py::arg("n_expert"), py::arg("want_inv") = true);
   m.def("route_static", &route_static, py::arg("gate"), py::arg("n_expert"), py::arg("count"),
         py::arg("seg_off"), py::arg("pos"), py::arg("inv") = py::none());
-  m.def("grouped_linear_fwd", &grouped_linear_fwd, py::arg("x"), py::arg("seg_off"),
-        py::arg("weight"), py::arg("bias") = py::none());
+  m.def("grouped_linear_fwd", &grouped_linear_fwd_any, py::arg("x"), py::arg("seg_off"),
+        py::arg("weight"), py::arg("bias") = py::none(), py::arg("with_gelu") = false);
   m.def("grouped_linear_bwd", &grouped_linear_bwd, py::arg("dy"), py::arg("x"), py::arg("seg_off"),
         py::arg("weight"), py::arg("need_bias") = true, py::arg("need_dx") = true,
         py::arg("need_dw") = true, py::arg("act_pre") = py::none());

@@ -29,6 +29,11 @@ struct GemmArgs {
   // and act_table the device table of gelu'(-|x|) (gelu_bwd_table()).
   const void* act_pre = nullptr;
   const float* act_table = nullptr;
+  // FWD on the bf16 matrix-core kernel only: if not null, act_out [n_rows, out_feat]
+  // receives gelu(y) next to y, through act_fwd_table, the device table of gelu(x)
+  // by 16-bit pattern of x (gelu_fwd_table()).
+  void* act_out = nullptr;
+  const uint16_t* act_fwd_table = nullptr;
 };
 
 // The part of the gelu'(-|x|) table the fused DGRAD epilogue keeps in LDS: the
@@ -42,6 +47,8 @@ constexpr int kActTabLdsOffset = 256 * (256 + 8) * 2;   // bytes from the start 
 
 // Device table of gelu'(-|x|) for a 16-bit dtype, built on first use (act.hip).
 int gelu_bwd_table(int dtype, hipStream_t s, const float** table);
+// Device table of gelu(x) by the 16-bit pattern of x (65536 results of the dtype).
+int gelu_fwd_table(int dtype, hipStream_t s, const uint16_t** table);
 
 // Virtual row-tile index space of the scalar kernel: expert e owns the tiles
 // from seg_off[e] / BM + e on (the starts are strictly increasing, so tiles

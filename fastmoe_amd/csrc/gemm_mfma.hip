@@ -735,6 +735,59 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
       (void*)(C + (int64_t)m0 * ldc + n0), (short)0, ((m_valid - 1) * ldc + n_valid) * 2,
       kRsrcFlags);
   const int c_off = n0 + pk * 8 < N ? (r0 * ldc + pk * 8) * 2 : (int)kOutOfRange;
+  // FWD with the activation fused in (g.act_out): the tile is written twice, as it
+  // is (the pre-activations the backward needs) and through the table of
+  // gelu(x) for 16-bit x, whose slice for 2^-28 <= |x| < 16 (both signs, 8192
+  // results) sits in LDS behind the staged tile; a pack with an argument outside
+  // that range (zeros, denormals, |x| >= 16, infinities, NaNs) is looked up in the
+  // full table in memory.
+  const bool fuse_fwd = MODE == GEMM_FWD && g.act_out != nullptr;
+  uint16_t* fwd_tab = smem + kActTabLdsOffset / 2;
+  static_assert(BM * kLdc * 2 <= kActTabLdsOffset, "the table sits behind the largest staged tile");
+  static_assert((kActTabBytes / 16) % NT == 0, "the table splits evenly over the threads");
+  constexpr int kTabPerThread = kActTabBytes / 16 / NT;
+  i32x4_t tab_regs[kTabPerThread];
+#pragma unroll
+  for (int i = 0; i < kTabPerThread; ++i) tab_regs[i] = i32x4_t{0, 0, 0, 0};
+  __amdgpu_buffer_rsrc_t a_rsrc = c_rsrc;
+  if (MODE == GEMM_FWD && fuse_fwd) {
+    // 16-byte piece L of the slice: 8 results from pattern 0x3180 + 8 L on, the
+    // second half of the pieces from 0xB180 on (the negative arguments)
+    constexpr int kHalfPieces = kActTabBytes / 16 / 2;
+#pragma unroll
+    for (int i = 0; i < kTabPerThread; ++i) {
+      const int piece = tid + i * NT;
+      const int first = piece < kHalfPieces ? kActTabFirst + 8 * piece
+                                            : 0x8000 + kActTabFirst + 8 * (piece - kHalfPieces);
+      tab_regs[i] = *reinterpret_cast<const i32x4_t*>(g.act_fwd_table + first);
+    }
+    a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)((T*)g.act_out + (int64_t)row0 * ldc + (int64_t)m0 * ldc + n0), (short)0,
+        ((m_valid - 1) * ldc + n_valid) * 2, kRsrcFlags);
+  }
+  // gelu of the 8 values of a pack
+  auto act_of = [&](i32x4_t pre) -> i32x4_t {
+    i32x4_t out;
+    uint32_t seen = 0;
+#pragma unroll
+    for (int wd = 0; wd < 4; ++wd) {
+      const uint32_t pw = (uint32_t)pre[wd];
+      const uint32_t t0 = (pw & 0x7fffu) - kActTabFirst, t1 = ((pw >> 16) & 0x7fffu) - kActTabFirst;
+      seen |= t0 | t1;
+      const uint32_t r0v = fwd_tab[t0 | ((pw >> 3) & 0x1000u)];
+      const uint32_t r1v = fwd_tab[t1 | ((pw >> 19) & 0x1000u)];
+      out[wd] = (int)(r0v | (r1v << 16));
+    }
+    if (__builtin_amdgcn_ballot_w64(seen >= (uint32_t)kActTabCount) != 0) {
+#pragma unroll
+      for (int wd = 0; wd < 4; ++wd) {
+        const uint32_t pw = (uint32_t)pre[wd];
+        out[wd] = (int)((uint32_t)g.act_fwd_table[pw & 0xffffu] |
+                        ((uint32_t)g.act_fwd_table[pw >> 16] << 16));
+      }
+    }
+    return out;
+  };
   // The upper half of every wave's rows is staged while the packs of the lower
   // half are on their way out: the stores leave at the address unit's pace (about
   // 30 cycles per wave instruction), the staging is conversion work for the vector
@@ -751,11 +804,16 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
       constexpr int b = decltype(b_tag)::value;
       stage_block(std::integral_constant<int, b % (TM / 2)>{}, std::integral_constant<int, b / (TM / 2)>{});
     });
+    if (MODE == GEMM_FWD && fuse_fwd) {
+#pragma unroll
+      for (int i = 0; i < kTabPerThread; ++i)
+        reinterpret_cast<i32x4_t*>(fwd_tab)[tid + i * NT] = tab_regs[i];
+    }
     __syncthreads();
     // Every pack gets registers of its own: a store holds its data registers
     // until memory has acknowledged it, so a register reused for a later pack
     // would make that pack wait for a full store round trip.
-    i32x4_t v[kSteps];
+    i32x4_t v[kSteps], w[kHalf];
 #pragma unroll
     for (int s2 = 0; s2 < kHalf; ++s2)
       v[s2] = *reinterpret_cast<const i32x4_t*>(sp + step_of(0, s2) * kRowsPerStep * kLdc);
@@ -763,6 +821,11 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
       constexpr int s2 = decltype(s_tag)::value;
       __builtin_amdgcn_raw_buffer_store_b128(
           v[s2], c_rsrc, c_off + step_of(0, s2) * kRowsPerStep * ldc * 2, 0, 0);
+      if (MODE == GEMM_FWD && fuse_fwd) {
+        w[s2] = act_of(v[s2]);
+        __builtin_amdgcn_raw_buffer_store_b128(
+            w[s2], a_rsrc, c_off + step_of(0, s2) * kRowsPerStep * ldc * 2, 0, 0);
+      }
       constexpr int b_lo = s2 * kBlocks / kHalf, b_hi = (s2 + 1) * kBlocks / kHalf;
       static_for<b_hi - b_lo>([&](auto d_tag) {
         constexpr int b = b_lo + decltype(d_tag)::value;
@@ -776,23 +839,40 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
     for (int s2 = 0; s2 < kHalf; ++s2)
       v[kHalf + s2] = *reinterpret_cast<const i32x4_t*>(sp + step_of(1, s2) * kRowsPerStep * kLdc);
 #pragma unroll
-    for (int s2 = 0; s2 < kHalf; ++s2)
+    for (int s2 = 0; s2 < kHalf; ++s2) {
       __builtin_amdgcn_raw_buffer_store_b128(
           v[kHalf + s2], c_rsrc, c_off + step_of(1, s2) * kRowsPerStep * ldc * 2, 0, 0);
+      if (MODE == GEMM_FWD && fuse_fwd) {
+        w[s2] = act_of(v[kHalf + s2]);
+        __builtin_amdgcn_raw_buffer_store_b128(
+            w[s2], a_rsrc, c_off + step_of(1, s2) * kRowsPerStep * ldc * 2, 0, 0);
+      }
+    }
   } else {
     static_for<TM * TN>([&](auto b_tag) {
       constexpr int b = decltype(b_tag)::value;
       stage_block(std::integral_constant<int, b % TM>{}, std::integral_constant<int, b / TM>{});
     });
+    if (MODE == GEMM_FWD && fuse_fwd) {
+#pragma unroll
+      for (int i = 0; i < kTabPerThread; ++i)
+        reinterpret_cast<i32x4_t*>(fwd_tab)[tid + i * NT] = tab_regs[i];
+    }
     __syncthreads();
-    i32x4_t v[kSteps];
+    i32x4_t v[kSteps], w[kSteps];
 #pragma unroll
     for (int u = 0; u < kSteps; ++u)
       v[u] = *reinterpret_cast<const i32x4_t*>(sp + u * kRowsPerStep * kLdc);
 #pragma unroll
-    for (int u = 0; u < kSteps; ++u)
+    for (int u = 0; u < kSteps; ++u) {
       __builtin_amdgcn_raw_buffer_store_b128(v[u], c_rsrc, c_off + u * kRowsPerStep * ldc * 2, 0,
                                              0);
+      if (MODE == GEMM_FWD && fuse_fwd) {
+        w[u] = act_of(v[u]);
+        __builtin_amdgcn_raw_buffer_store_b128(w[u], a_rsrc, c_off + u * kRowsPerStep * ldc * 2,
+                                               0, 0);
+      }
+    }
   }
 }
 
@@ -1683,8 +1763,15 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
   constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
+  // a forward launch with the activation fused in keeps the table slice behind the
+  // place of the largest staged tile, whatever its own tile shape
+  constexpr size_t act_bytes = (size_t)kActTabLdsOffset + kActTabBytes;
+  constexpr size_t lds_max =
+      MODE == GEMM_FWD && act_bytes > lds_bytes ? act_bytes : lds_bytes;
+  static_assert(lds_max + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
+  const size_t lds_launch = MODE == GEMM_FWD && g.act_out ? lds_max : lds_bytes;
   auto kern = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, NS, MODE>;
-  FMOE_SET_DYNAMIC_LDS_ONCE(kern, lds_bytes);
+  FMOE_SET_DYNAMIC_LDS_ONCE(kern, lds_max);
   int tiles_n, tiles_m;
   int64_t blocks;
   if (MODE == GEMM_WGRAD) {
@@ -1706,7 +1793,7 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   FMOE_REQUIRE(blocks < ((int64_t)1 << 31), FMOE_ERR_UNSUPPORTED,
                "grouped GEMM: too many tiles");
   if (blocks == 0) return FMOE_OK;
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NT), lds_bytes, s, g,
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NT), lds_launch, s, g,
                      tiles_n, tiles_m);
   FMOE_LAUNCH_CHECK("gemm_mfma");
   return FMOE_OK;

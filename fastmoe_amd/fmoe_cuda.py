@@ -347,8 +347,12 @@ def route_static(gate: torch.Tensor, n_expert: int, count: torch.Tensor, seg_off
 
 
 def grouped_linear_fwd(x: torch.Tensor, seg_off: torch.Tensor, weight: torch.Tensor,
-                       bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """y[seg_e] = x[seg_e] @ weight[e].T + bias[e] with device-side seg_off."""
+                       bias: Optional[torch.Tensor] = None, with_gelu: bool = False):
+    """y[seg_e] = x[seg_e] @ weight[e].T + bias[e] with device-side seg_off.
+
+    with_gelu: returns (y, gelu(y)), the exact GELU applied to the rounded y, written
+    by the same output tiles where the library can (rows behind seg_off[E] are left
+    as allocated in both)."""
     _dev(x, "x")
     _dev(weight, "weight", x.dtype)
     _dev(seg_off, "seg_off", torch.int32)
@@ -361,6 +365,16 @@ def grouped_linear_fwd(x: torch.Tensor, seg_off: torch.Tensor, weight: torch.Ten
         _need(tuple(bias.shape) == (e, out_f), "bias must be [E, out]")
     dt = _dt(x, "x")
     y = torch.empty((x.shape[0], out_f), dtype=x.dtype, device=x.device)
+    if with_gelu:
+        y_act = torch.empty_like(y)
+        with _launch(x, "grouped_linear_fwd_act"):
+            _lib.check(
+                _L.fmoe_grouped_linear_fwd_act(x.data_ptr(), weight.data_ptr(), _ptr(bias),
+                                               seg_off.data_ptr(), y.data_ptr(),
+                                               y_act.data_ptr(), x.shape[0], in_f, out_f, e,
+                                               dt, _stream(x)),
+                "grouped_linear_fwd_act")
+        return y, y_act
     with _launch(x, "grouped_linear_fwd"):
         _lib.check(
             _L.fmoe_grouped_linear_fwd(x.data_ptr(), weight.data_ptr(), _ptr(bias),
@@ -555,11 +569,17 @@ def set_gemm_path(path: int) -> None:
     _lib.check(_L.fmoe_set_gemm_path(path), "set_gemm_path")
 
 
-def _hooked(name, fn):
+def _hooked(op_name, fn):
     """A compiled operator that reports to `profile_hook` the way the ctypes ones do."""
 
     def op(*args, **kwargs):
-        if profile_hook is None or (profile_only is not None and name not in profile_only):
+        if profile_hook is None:
+            return fn(*args, **kwargs)
+        name = op_name
+        if name == "grouped_linear_fwd" and (kwargs.get("with_gelu") or
+                                             (len(args) > 4 and args[4])):
+            name = "grouped_linear_fwd_act"
+        if profile_only is not None and name not in profile_only:
             return fn(*args, **kwargs)
         first = next((a for a in args if isinstance(a, torch.Tensor) and a.is_cuda), None)
         if first is None:
@@ -572,7 +592,7 @@ def _hooked(name, fn):
         profile_hook(name, start, end)
         return out
 
-    op.__name__ = name
+    op.__name__ = op_name
     op.__doc__ = fn.__doc__
     return op
 

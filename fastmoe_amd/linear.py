@@ -43,6 +43,35 @@ class MOELinear(Function):
         return dx, None, dw, db
 
 
+class MOELinearGelu(Function):
+    r"""A grouped linear layer that returns its output twice: as it is (the
+    pre-activations, the differentiable result) and through the exact GELU, written by
+    the same output tiles where the library can (bf16 on the matrix cores).  The
+    second result carries no gradient of its own: it is meant for MOEGeluLinear,
+    whose backward returns the gradient with respect to the pre-activations."""
+
+    @staticmethod
+    def forward(ctx, global_input_buf, fwd_expert_count, weight, bias=None):
+        x = global_input_buf.contiguous()
+        seg_off = _segments(fwd_expert_count, x.device)
+        pre, act = fmoe_cuda.grouped_linear_fwd(
+            x, seg_off, weight.contiguous(), None if bias is None else bias.contiguous(),
+            with_gelu=True)
+        ctx.save_for_backward(x, seg_off, weight, bias)
+        ctx.mark_non_differentiable(act)
+        return pre, act
+
+    @staticmethod
+    def backward(ctx, grad_pre, _grad_act):
+        (x, seg_off, weight, bias) = ctx.saved_tensors
+        need_dx, _, need_dw, need_db = ctx.needs_input_grad
+        need_db = need_db and torch.is_tensor(bias)
+        dx, dw, db = fmoe_cuda.grouped_linear_bwd(
+            grad_pre.contiguous(), x, seg_off, weight.contiguous(),
+            need_bias=need_db, need_dx=need_dx, need_dw=need_dw)
+        return dx, None, dw, db
+
+
 class MOEGeluLinear(Function):
     r"""`linear(gelu(pre))` as one autograd node: the activation between the two
     expert layers and the second layer (fmoe/transformer.py:28-31 for
@@ -52,10 +81,11 @@ class MOEGeluLinear(Function):
     dY W to memory for a separate activation kernel to read back."""
 
     @staticmethod
-    def forward(ctx, pre, fwd_expert_count, weight, bias=None):
+    def forward(ctx, pre, fwd_expert_count, weight, bias=None, act=None):
         pre = pre.contiguous()
         seg_off = _segments(fwd_expert_count, pre.device)
-        act = fmoe_cuda.gelu_fwd(pre, seg_off[-1:])      # rows past the last segment are dead
+        if act is None:   # (MOELinearGelu hands over gelu(pre) with the pre-activations)
+            act = fmoe_cuda.gelu_fwd(pre, seg_off[-1:])  # rows past the last segment are dead
         out = fmoe_cuda.grouped_linear_fwd(act, seg_off, weight.contiguous(),
                                            None if bias is None else bias.contiguous())
         ctx.save_for_backward(pre, act, seg_off, weight, bias)
@@ -64,12 +94,12 @@ class MOEGeluLinear(Function):
     @staticmethod
     def backward(ctx, grad_out):
         (pre, act, seg_off, weight, bias) = ctx.saved_tensors
-        need_dx, _, need_dw, need_db = ctx.needs_input_grad
+        need_dx, _, need_dw, need_db = ctx.needs_input_grad[:4]
         need_db = need_db and torch.is_tensor(bias)
         dpre, dw, db = fmoe_cuda.grouped_linear_bwd(
             grad_out.contiguous(), act, seg_off, weight.contiguous(),
             need_bias=need_db, need_dx=need_dx, need_dw=need_dw, act_pre=pre)
-        return dpre, None, dw, db
+        return dpre, None, dw, db, None
 
 
 def is_exact_gelu(activation, x: torch.Tensor) -> bool:
@@ -86,6 +116,19 @@ def act_linear(activation, pre, fwd_expert_count, weight, bias):
     live = fwd_expert_count.seg_off[-1:] if isinstance(fwd_expert_count, SegmentTable) else None
     x = apply_activation(activation, pre, live)
     return MOELinear.apply(x.type_as(weight), fwd_expert_count, weight, bias)
+
+
+def linear_act_linear(activation, inp, fwd_expert_count, weight1, bias1, weight2, bias2):
+    r"""The reference's expert, `h4toh(activation(htoh4(inp)))` (fmoe/transformer.py:
+    25-33), over the experts' row segments.  With torch.nn.GELU() the activation is
+    written by the first layer's output tiles and differentiated inside the second
+    layer's backward tiles."""
+    x = inp.type_as(weight1)
+    if is_exact_gelu(activation, x) and weight1.dtype == weight2.dtype:
+        pre, act = MOELinearGelu.apply(x, fwd_expert_count, weight1, bias1)
+        return MOEGeluLinear.apply(pre, fwd_expert_count, weight2, bias2, act)
+    pre = MOELinear.apply(x, fwd_expert_count, weight1, bias1)
+    return act_linear(activation, pre, fwd_expert_count, weight2, bias2)
 
 
 class FMoELinear(nn.Module):

@@ -6,7 +6,7 @@ import torch.nn as nn
 
 from .functions import SegmentTable
 from .layers import FMoE
-from .linear import FMoELinear, MOELinear, act_linear
+from .linear import FMoELinear, MOELinear, act_linear, linear_act_linear
 
 
 class _LinearView:
@@ -57,11 +57,17 @@ class _Expert(nn.Module):
         self.activation = activation
 
     def forward(self, inp, fwd_expert_count):
-        x = self.htoh4(inp, fwd_expert_count)
-        # activation and second layer as one node: the activation's backward runs
-        # inside the second layer's backward kernel
-        return act_linear(self.activation, x, fwd_expert_count, self.h4toh.weight,
-                          self.h4toh.bias)
+        if any(m._forward_hooks or m._forward_pre_hooks for m in (self.htoh4, self.h4toh)):
+            # somebody watches the two linear modules: call them as modules
+            x = self.htoh4(inp, fwd_expert_count)
+            if self.h4toh._forward_hooks or self.h4toh._forward_pre_hooks:
+                return self.h4toh(self.activation(x), fwd_expert_count)
+            return act_linear(self.activation, x, fwd_expert_count, self.h4toh.weight,
+                              self.h4toh.bias)
+        # the activation is written by the first layer's output tiles, and its
+        # backward runs inside the second layer's backward kernel
+        return linear_act_linear(self.activation, inp, fwd_expert_count, self.htoh4.weight,
+                                 self.htoh4.bias, self.h4toh.weight, self.h4toh.bias)
 
     def __len__(self):
         return self.htoh4.num_expert
@@ -106,8 +112,7 @@ class _Expert(nn.Module):
         first = experts[0]
         w1, b1 = cat(lambda e: e.htoh4.weight), cat(lambda e: e.htoh4.bias)
         w2, b2 = cat(lambda e: e.h4toh.weight), cat(lambda e: e.h4toh.bias)
-        x = MOELinear.apply(inp.type_as(w1), segments, w1, b1)
-        return act_linear(first.activation, x, segments, w2, b2)
+        return linear_act_linear(first.activation, inp, segments, w1, b1, w2, b2)
 
 
 class FMoETransformerMLP(FMoE):

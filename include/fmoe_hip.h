@@ -251,6 +251,21 @@ int fmoe_grouped_linear_bwd(const void* dy, const void* x, const void* w,
                             void* stream);
 
 /*
+ * Forward of the first layer of the reference's expert with its activation
+ * (fmoe/transformer.py:25-33: htoh4 -> activation): y as fmoe_grouped_linear_fwd
+ * writes it (the pre-activations, which the backward needs) and y_act = gelu(y),
+ * the exact GELU of torch.nn.GELU().  Where the bf16 matrix-core kernel runs, both
+ * leave the same output tiles (the activation kernel's own table of gelu(x) for
+ * 16-bit x, applied to the rounded y: the same bits as fmoe_gelu_fwd over y); for
+ * other dtypes and shapes the entry point runs that kernel behind the GEMM.  Rows of
+ * y_act behind seg_off[n_expert] are left untouched, like those of y.
+ */
+int fmoe_grouped_linear_fwd_act(const void* x, const void* w, const void* bias,
+                                const int32_t* seg_off, void* y, void* y_act,
+                                int64_t n_rows, int64_t in_feat, int64_t out_feat,
+                                int64_t n_expert, int dtype, void* stream);
+
+/*
  * fmoe_grouped_linear_bwd for a layer whose input is act = gelu(act_pre), with
  * the activation's backward folded in: dx = (dY[seg_e] * W_e) .* gelu'(act_pre),
  * x being act (dW is unchanged).  act_pre is [n_rows, in_feat].  bf16 on the
