@@ -59,10 +59,14 @@ class MOELinearGelu(Function):
             with_gelu=True)
         ctx.save_for_backward(x, seg_off, weight, bias)
         ctx.mark_non_differentiable(act)
+        # (or autograd would fill a zero tensor of act's size for it at every backward)
+        ctx.set_materialize_grads(False)
         return pre, act
 
     @staticmethod
     def backward(ctx, grad_pre, _grad_act):
+        if grad_pre is None:
+            return None, None, None, None
         (x, seg_off, weight, bias) = ctx.saved_tensors
         need_dx, _, need_dw, need_db = ctx.needs_input_grad
         need_db = need_db and torch.is_tensor(bias)

@@ -130,13 +130,25 @@ def test_expert_module_runs_no_activation_kernel_of_its_own(dt):
         y.backward(dy)
         return [y.detach(), xi.grad] + [p.grad.clone() for p in ex.parameters()]
 
-    seen = []
+    from fastmoe_amd.linear import MOELinearGelu
+
+    seen, act_grads = [], []
+    inner = MOELinearGelu.backward
+
+    def spy(ctx, grad_pre, grad_act):
+        act_grads.append(grad_act)
+        return inner(ctx, grad_pre, grad_act)
+
     fmoe_cuda.profile_hook = lambda name, a, b: seen.append(name)
+    MOELinearGelu.backward = staticmethod(spy)
     try:
         got = run(lambda xi: ex(xi, counts))
     finally:
         fmoe_cuda.profile_hook = None
+        MOELinearGelu.backward = staticmethod(inner)
     assert "gelu_fwd" not in seen and "gelu_bwd" not in seen
+    # no zero tensor of the activation's size is made for the output that carries no gradient
+    assert act_grads == [None]
     assert seen.count("grouped_linear_fwd_act") == 1 and seen.count("grouped_linear_fwd") == 1
     assert seen.count("grouped_linear_bwd") == 2
 
