@@ -57,10 +57,10 @@ PEAK = {"hbm": 8.0e12, "bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 # whose traffic is known (FETCH_SIZE x 1.035 on cfg2 and cfg5, x 0.998 on cfg4;
 # WRITE_SIZE x 1.000).  Only the workloads that were measured have an entry.
 MEASURED_TRAFFIC = {
-    ("cfg2", "grouped_linear_bwd"): (310.6 + 222.2) * 2 ** 20,
-    ("cfg2", "grouped_linear_fwd"): (154.6 + 80.0) * 2 ** 20,
-    ("cfg4", "grouped_linear_bwd"): (5988.2 + 1564.9) * 2 ** 20,
-    ("cfg4", "grouped_linear_fwd"): (2919.1 + 576.0) * 2 ** 20,
+    ("cfg2", "grouped_linear_bwd"): (310.4 + 213.1) * 2 ** 20,
+    ("cfg2", "grouped_linear_fwd"): (155.0 + 144.0) * 2 ** 20,
+    ("cfg4", "grouped_linear_bwd"): (5968.4 + 1507.1) * 2 ** 20,
+    ("cfg4", "grouped_linear_fwd"): (2921.7 + 1024.0) * 2 ** 20,
     ("cfg5", "grouped_linear_bwd"): (1247.1 + 961.3) * 2 ** 20,
     ("cfg5", "grouped_linear_fwd"): (811.3 + 216.0) * 2 ** 20,
 }
