@@ -9,7 +9,11 @@ namespace fmoe {
 //   FWD    Y[seg]  = X[seg]  * W_e^T (+ b_e)   M = rows, N = out,  K = in
 //   DGRAD  dX[seg] = dY[seg] * W_e             M = rows, N = in,   K = out
 //   WGRAD  dW_e    = dY[seg]^T * X[seg]        M = out,  N = in,   K = rows
-enum GemmMode { GEMM_FWD = 0, GEMM_DGRAD = 1, GEMM_WGRAD = 2 };
+enum GemmMode { GEMM_FWD = 0, GEMM_DGRAD = 1, GEMM_WGRAD = 2,
+                // FWD with GemmArgs::act_out: a kernel of its own inside the bf16
+                // matrix-core family (callers pass GEMM_FWD and set act_out)
+                GEMM_FWD_ACT = 3 };
+constexpr bool is_fwd(int mode) { return mode == GEMM_FWD || mode == GEMM_FWD_ACT; }
 
 struct GemmArgs {
   const void* a;        // FWD: x      DGRAD: dy     WGRAD: dy

@@ -369,7 +369,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   constexpr int NW = WM * WN;
   constexpr int NT = NW * 64;
   constexpr bool A_KC = MODE != GEMM_WGRAD;
-  constexpr bool B_KC = MODE == GEMM_FWD;
+  constexpr bool B_KC = is_fwd(MODE);
   constexpr int TM = BM / WM / 16, TN = BN / WN / 16;   // 16x16 blocks of a wave
   static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0 && BK % 32 == 0, "tile shape");
   static_assert((NS >= 4 && NS <= 8) || (NS == 2 && BK == 64), "LDS stages");
@@ -392,7 +392,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   int M, N, K, lda, ldb, ldc;
   const uint16_t *A, *B;
   T* C;
-  if (MODE == GEMM_FWD) {
+  if (is_fwd(MODE)) {
     M = cnt; N = out_f; K = in_f;
     A = (const uint16_t*)g.a + (int64_t)row0 * in_f;        lda = in_f;
     B = (const uint16_t*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
@@ -684,7 +684,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   // 8-byte writes of 16 rows x 2 column groups, the 32 lanes served together,
   // spread over the banks) and leaves as 16-byte packs: one wave instruction
   // then stores whole 512-byte row segments.
-  const T* bias = (MODE == GEMM_FWD && g.bias)
+  const T* bias = (is_fwd(MODE) && g.bias)
                       ? (const T*)g.bias + (int64_t)e * out_f : nullptr;
   struct alignas(8) Out4 { T v[4]; };
   constexpr int kLdc = BN + 8;   // elements per staged row
@@ -693,7 +693,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   // are: adding a zero would cost an instruction per value, which the compiler may
   // not drop because of -0.  ONE code path: two variants of this loop made the
   // register allocator shuffle the accumulators inside the K loop.)
-  constexpr bool kBias = MODE == GEMM_FWD;
+  constexpr bool kBias = is_fwd(MODE);
   float bv[TN][4];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -741,7 +741,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   // results) sits in LDS behind the staged tile; a pack with an argument outside
   // that range (zeros, denormals, |x| >= 16, infinities, NaNs) is looked up in the
   // full table in memory.
-  const bool fuse_fwd = MODE == GEMM_FWD && g.act_out != nullptr;
+  constexpr bool fuse_fwd = MODE == GEMM_FWD_ACT;
   uint16_t* fwd_tab = smem + kActTabLdsOffset / 2;
   static_assert(BM * kLdc * 2 <= kActTabLdsOffset, "the table sits behind the largest staged tile");
   static_assert((kActTabBytes / 16) % NT == 0, "the table splits evenly over the threads");
@@ -750,7 +750,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
 #pragma unroll
   for (int i = 0; i < kTabPerThread; ++i) tab_regs[i] = i32x4_t{0, 0, 0, 0};
   __amdgpu_buffer_rsrc_t a_rsrc = c_rsrc;
-  if (MODE == GEMM_FWD && fuse_fwd) {
+  if constexpr (fuse_fwd) {
     // 16-byte piece L of the slice: 8 results from pattern 0x3180 + 8 L on, the
     // second half of the pieces from 0xB180 on (the negative arguments)
     constexpr int kHalfPieces = kActTabBytes / 16 / 2;
@@ -804,7 +804,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
       constexpr int b = decltype(b_tag)::value;
       stage_block(std::integral_constant<int, b % (TM / 2)>{}, std::integral_constant<int, b / (TM / 2)>{});
     });
-    if (MODE == GEMM_FWD && fuse_fwd) {
+    if constexpr (fuse_fwd) {
 #pragma unroll
       for (int i = 0; i < kTabPerThread; ++i)
         reinterpret_cast<i32x4_t*>(fwd_tab)[tid + i * NT] = tab_regs[i];
@@ -821,7 +821,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
       constexpr int s2 = decltype(s_tag)::value;
       __builtin_amdgcn_raw_buffer_store_b128(
           v[s2], c_rsrc, c_off + step_of(0, s2) * kRowsPerStep * ldc * 2, 0, 0);
-      if (MODE == GEMM_FWD && fuse_fwd) {
+      if constexpr (fuse_fwd) {
         w[s2] = act_of(v[s2]);
         __builtin_amdgcn_raw_buffer_store_b128(
             w[s2], a_rsrc, c_off + step_of(0, s2) * kRowsPerStep * ldc * 2, 0, 0);
@@ -842,7 +842,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
     for (int s2 = 0; s2 < kHalf; ++s2) {
       __builtin_amdgcn_raw_buffer_store_b128(
           v[kHalf + s2], c_rsrc, c_off + step_of(1, s2) * kRowsPerStep * ldc * 2, 0, 0);
-      if (MODE == GEMM_FWD && fuse_fwd) {
+      if constexpr (fuse_fwd) {
         w[s2] = act_of(v[kHalf + s2]);
         __builtin_amdgcn_raw_buffer_store_b128(
             w[s2], a_rsrc, c_off + step_of(1, s2) * kRowsPerStep * ldc * 2, 0, 0);
@@ -853,7 +853,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
       constexpr int b = decltype(b_tag)::value;
       stage_block(std::integral_constant<int, b % TM>{}, std::integral_constant<int, b / TM>{});
     });
-    if (MODE == GEMM_FWD && fuse_fwd) {
+    if constexpr (fuse_fwd) {
 #pragma unroll
       for (int i = 0; i < kTabPerThread; ++i)
         reinterpret_cast<i32x4_t*>(fwd_tab)[tid + i * NT] = tab_regs[i];
@@ -867,7 +867,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
     for (int u = 0; u < kSteps; ++u) {
       __builtin_amdgcn_raw_buffer_store_b128(v[u], c_rsrc, c_off + u * kRowsPerStep * ldc * 2, 0,
                                              0);
-      if (MODE == GEMM_FWD && fuse_fwd) {
+      if constexpr (fuse_fwd) {
         w[u] = act_of(v[u]);
         __builtin_amdgcn_raw_buffer_store_b128(w[u], a_rsrc, c_off + u * kRowsPerStep * ldc * 2,
                                                0, 0);
@@ -885,7 +885,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   constexpr int NW = WM * WN;
   constexpr int NT = NW * 64;
   constexpr bool A_KC = MODE != GEMM_WGRAD;
-  constexpr bool B_KC = MODE == GEMM_FWD;
+  constexpr bool B_KC = is_fwd(MODE);
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0 && BK % 16 == 0, "tile shape");
   static_assert((NS >= 4 && NS <= 8) || (NS == 2 && BK == 64), "LDS stages");
@@ -908,7 +908,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   int M, N, K, lda, ldb, ldc;
   const uint16_t *A, *B;
   T* C;
-  if (MODE == GEMM_FWD) {
+  if (is_fwd(MODE)) {
     M = cnt; N = out_f; K = in_f;
     A = (const uint16_t*)g.a + (int64_t)row0 * in_f;        lda = in_f;
     B = (const uint16_t*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
@@ -1189,7 +1189,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   // The tile goes through LDS (row-major, rows padded by 16 bytes so that the
   // 8-byte writes of 32 rows spread over the banks) and leaves as 16-byte packs:
   // one wave instruction then stores whole 512-byte row segments.
-  const T* bias = (MODE == GEMM_FWD && g.bias)
+  const T* bias = (is_fwd(MODE) && g.bias)
                       ? (const T*)g.bias + (int64_t)e * out_f : nullptr;
   struct alignas(8) Out4 { T v[4]; };
   constexpr int kLdc = BN + 8;   // elements per staged row
@@ -1214,7 +1214,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   // (only the forward product has a bias; elsewhere the sums are rounded as they
   // are: adding a zero would cost an instruction per value, which the compiler may
   // not drop because of -0)
-  constexpr bool kBias = MODE == GEMM_FWD;
+  constexpr bool kBias = is_fwd(MODE);
   // 4 columns of block (i, j), column group q, rounded, into the staged tile
   auto stage_block = [&](auto i_tag, auto j_tag, auto q_tag) {
     constexpr int i = decltype(i_tag)::value, j = decltype(j_tag)::value;
@@ -1389,7 +1389,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
 // FWD 1.29-1.31 vs 1.24-1.26 PFLOP/s with 16x16x32, DGRAD 1.21 vs 1.35 and
 // WGRAD 1.24 vs 1.27 the other way round.
 #ifndef FMOE_MFMA16_MODES
-#define FMOE_MFMA16_MODES (1 << GEMM_FWD)
+#define FMOE_MFMA16_MODES ((1 << GEMM_FWD) | (1 << GEMM_FWD_ACT))
 #endif
 template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, int MODE>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint16_t* smem, TileRows where,
@@ -1443,7 +1443,7 @@ __device__ __forceinline__ void edge_aware_tile(const GemmArgs& g, uint16_t* sme
                                                 int n_tile) {
   const int n0 = n_tile * BN;
   if constexpr (BM == 256 && BN == 256 && WM == 2 && WN == 2) {
-    const int n_total = MODE == GEMM_FWD ? g.out_feat : g.in_feat;
+    const int n_total = is_fwd(MODE) ? g.out_feat : g.in_feat;
     if (n_total - n0 <= BN / 2) {
       gemm_tile<T, BM, BN / 2, BK, WM, WN, NS, MODE>(g, smem, where, n0);
       return;
@@ -1469,7 +1469,7 @@ constexpr int kNarrowMax = 128;
 constexpr int kNarrowMinK = 2048;
 template <int BM, int BN, int MODE>
 constexpr int narrow_factor() {
-  return (BM == 256 && BN == 256 && MODE != GEMM_WGRAD) ? (MODE == GEMM_FWD ? 4 : 2) : 1;
+  return (BM == 256 && BN == 256 && MODE != GEMM_WGRAD) ? (is_fwd(MODE) ? 4 : 2) : 1;
 }
 
 // Runs the remainder tile at rows [where.m0, where.cnt) of its expert; n_tile
@@ -1671,7 +1671,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
   constexpr int kF = kSmall ? narrow_factor<BM, BN, MODE>() : 1;
   const int wide_s = rows.rows_s * tiles_n;
   const bool narrow = kF > 1 && wide_s <= kNarrowMax &&
-                      (MODE == GEMM_FWD ? g.in_feat : g.out_feat) >= kNarrowMinK;
+                      (is_fwd(MODE) ? g.in_feat : g.out_feat) >= kNarrowMinK;
   const int cols_s = narrow ? tiles_n * kF : tiles_n;
   const int live_f = rows.rows_f * tiles_n, live = live_f + rows.rows_s * cols_s;
   if (live == 0) return;
@@ -1753,7 +1753,7 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   constexpr int NW = WM * WN;
   constexpr int NT = NW * 64;
   using ATile = DmaTile<BM, BK, NW, MODE != GEMM_WGRAD>;
-  using BTile = DmaTile<BN, BK, NW, MODE == GEMM_FWD>;
+  using BTile = DmaTile<BN, BK, NW, is_fwd(MODE)>;
   constexpr size_t pipe_bytes = NS * (ATile::kBytes + BTile::kBytes);
   // staged output tile (+ the activation table of a fused DGRAD epilogue)
   constexpr size_t out_bytes =
@@ -1767,9 +1767,9 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   // place of the largest staged tile, whatever its own tile shape
   constexpr size_t act_bytes = (size_t)kActTabLdsOffset + kActTabBytes;
   constexpr size_t lds_max =
-      MODE == GEMM_FWD && act_bytes > lds_bytes ? act_bytes : lds_bytes;
+      MODE == GEMM_FWD_ACT && act_bytes > lds_bytes ? act_bytes : lds_bytes;
   static_assert(lds_max + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
-  const size_t lds_launch = MODE == GEMM_FWD && g.act_out ? lds_max : lds_bytes;
+  constexpr size_t lds_launch = lds_max;
   auto kern = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, NS, MODE>;
   FMOE_SET_DYNAMIC_LDS_ONCE(kern, lds_max);
   int tiles_n, tiles_m;
@@ -1779,7 +1779,7 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
     tiles_m = ceil_div(g.out_feat, BM);
     blocks = (int64_t)tiles_n * tiles_m * g.n_expert;
   } else {
-    tiles_n = ceil_div(MODE == GEMM_FWD ? g.out_feat : g.in_feat, BN);
+    tiles_n = ceil_div(is_fwd(MODE) ? g.out_feat : g.in_feat, BN);
     // at most n_rows / BM whole tiles plus, per expert, one more BM tile or
     // one remainder tile
     tiles_m = (int)(g.n_rows / BM) + g.n_expert;
@@ -1809,9 +1809,9 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
 template <int MODE>
 static int pick_tile(const GemmArgs& g) {
   if (g.tile >= 1 && g.tile <= 4) return g.tile;
-  const int64_t N = MODE == GEMM_FWD ? g.out_feat : g.in_feat;
+  const int64_t N = is_fwd(MODE) ? g.out_feat : g.in_feat;
   const int64_t K = MODE == GEMM_WGRAD ? g.n_rows / g.n_expert
-                                       : (MODE == GEMM_FWD ? g.in_feat : g.out_feat);
+                                       : (is_fwd(MODE) ? g.in_feat : g.out_feat);
   auto cost = [&](int bm, int bn, double us_per_slice, int blocks_per_cu) -> double {
     const int64_t tiles = MODE == GEMM_WGRAD
         ? (int64_t)g.n_expert * ceil_div(g.out_feat, bm) * ceil_div(g.in_feat, bn)
@@ -1843,7 +1843,13 @@ static int launch_mode(const GemmArgs& g, hipStream_t s) {
 template <typename T>
 static int launch_t(int mode, const GemmArgs& g, hipStream_t s) {
   switch (mode) {
-    case GEMM_FWD: return launch_mode<T, GEMM_FWD>(g, s);
+    case GEMM_FWD:
+      if constexpr (std::is_same<T, __hip_bfloat16>::value) {
+        if (g.act_out) return launch_mode<T, GEMM_FWD_ACT>(g, s);
+      }
+      FMOE_REQUIRE(g.act_out == nullptr, FMOE_ERR_UNSUPPORTED,
+                   "grouped GEMM: the fused activation is a bf16 kernel");
+      return launch_mode<T, GEMM_FWD>(g, s);
     case GEMM_DGRAD: return launch_mode<T, GEMM_DGRAD>(g, s);
     default: return launch_mode<T, GEMM_WGRAD>(g, s);
   }
