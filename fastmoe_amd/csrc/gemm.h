@@ -12,8 +12,11 @@ namespace fmoe {
 enum GemmMode { GEMM_FWD = 0, GEMM_DGRAD = 1, GEMM_WGRAD = 2,
                 // FWD with GemmArgs::act_out: a kernel of its own inside the bf16
                 // matrix-core family (callers pass GEMM_FWD and set act_out)
-                GEMM_FWD_ACT = 3 };
+                GEMM_FWD_ACT = 3,
+                // DGRAD with GemmArgs::act_pre, likewise (callers pass GEMM_DGRAD)
+                GEMM_DGRAD_ACT = 4 };
 constexpr bool is_fwd(int mode) { return mode == GEMM_FWD || mode == GEMM_FWD_ACT; }
+constexpr bool is_dgrad(int mode) { return mode == GEMM_DGRAD || mode == GEMM_DGRAD_ACT; }
 
 struct GemmArgs {
   const void* a;        // FWD: x      DGRAD: dy     WGRAD: dy

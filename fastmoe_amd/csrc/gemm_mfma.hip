@@ -397,7 +397,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
     A = (const uint16_t*)g.a + (int64_t)row0 * in_f;        lda = in_f;
     B = (const uint16_t*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
     C = (T*)g.c + (int64_t)row0 * out_f;                    ldc = out_f;
-  } else if (MODE == GEMM_DGRAD) {
+  } else if (is_dgrad(MODE)) {
     M = cnt; N = in_f; K = out_f;
     A = (const uint16_t*)g.a + (int64_t)row0 * out_f;       lda = out_f;
     B = (const uint16_t*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
@@ -913,7 +913,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
     A = (const uint16_t*)g.a + (int64_t)row0 * in_f;        lda = in_f;
     B = (const uint16_t*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
     C = (T*)g.c + (int64_t)row0 * out_f;                    ldc = out_f;
-  } else if (MODE == GEMM_DGRAD) {
+  } else if (is_dgrad(MODE)) {
     M = cnt; N = in_f; K = out_f;
     A = (const uint16_t*)g.a + (int64_t)row0 * out_f;       lda = out_f;
     B = (const uint16_t*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
@@ -1196,7 +1196,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   T* stage_c = reinterpret_cast<T*>(smem);
   // DGRAD with the activation's backward fused in: the slice of the gelu' table
   // goes into LDS behind the staged tile (its loads fly during the staging)
-  const bool fuse_act = MODE == GEMM_DGRAD && g.act_pre != nullptr;
+  constexpr bool fuse_act = MODE == GEMM_DGRAD_ACT;
   static_assert(BM * kLdc * 2 <= kActTabLdsOffset, "the table sits behind the largest staged tile");
   float* act_tab = reinterpret_cast<float*>(smem + kActTabLdsOffset / 2);
   // (an even split: a guarded load into the array would put it into scratch
@@ -1206,7 +1206,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   i32x4_t tab_regs[kTabPerThread];
 #pragma unroll
   for (int i = 0; i < kTabPerThread; ++i) tab_regs[i] = i32x4_t{0, 0, 0, 0};
-  if (MODE == GEMM_DGRAD && fuse_act) {
+  if constexpr (fuse_act) {
     const i32x4_t* src = reinterpret_cast<const i32x4_t*>(g.act_table + kActTabFirst);
 #pragma unroll
     for (int i = 0; i < kTabPerThread; ++i) tab_regs[i] = src[tid + i * NT];
@@ -1270,13 +1270,13 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   constexpr int kBlocksLo = kHalfRows * TN * 4, kBlocksHi = (TM - kHalfRows) * TN * 4;
   stage_blocks(std::integral_constant<int, 0>{}, std::integral_constant<int, kHalfRows>{},
                std::integral_constant<int, 0>{}, std::integral_constant<int, kBlocksLo>{});
-  if (MODE == GEMM_DGRAD && fuse_act) {
+  if constexpr (fuse_act) {
 #pragma unroll
     for (int i = 0; i < kTabPerThread; ++i)
       reinterpret_cast<i32x4_t*>(act_tab)[tid + i * NT] = tab_regs[i];
   }
   if constexpr (kOverlap) {
-    if (!(MODE == GEMM_DGRAD && fuse_act)) {
+    if constexpr (!fuse_act) {
       constexpr int kHalf = kSteps / 2;
       // store step of the s-th pack of half h
       auto step_of = [](int h, int s2) constexpr {
@@ -1316,7 +1316,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
                  std::integral_constant<int, kBlocksHi>{});
   }
   __syncthreads();
-  if (MODE == GEMM_DGRAD && fuse_act) {
+  if constexpr (fuse_act) {
     // dx = dH * gelu'(pre): the staged dH (already rounded to the storage type,
     // as a separate activation kernel would read it) times the table value of
     // the matching pre-activation pack, fetched through a descriptor with the
@@ -1697,19 +1697,21 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(GemmArgs g,
 // The tail of one product overlaps the head of the next instead of leaving CUs
 // idle between two launches.  gd / gw are the arguments the two products
 // would get on their own.
-template <typename T, int BM, int BN, int BK, int WM, int WN, int NS>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NS, bool ACT>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, GemmArgs gw,
                                                                int tiles_n_d, int tiles_n_w,
                                                                int tiles_m_w, int small_first) {
   constexpr int NW = WM * WN;
-  constexpr bool kSmall = has_small_tiles<BM, BN, GEMM_DGRAD>();
+  // dX with gelu' of the pre-activations applied in its tiles (gd.act_pre), or plain
+  constexpr int DMODE = ACT ? GEMM_DGRAD_ACT : GEMM_DGRAD;
+  constexpr bool kSmall = has_small_tiles<BM, BN, DMODE>();
   static_assert(!kSmall || NW == 4, "remainder tiles put 4 waves side by side");
   extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];
   __shared__ int s_owner[4], s_wave_sum[2 * NW];
 
   RowTiles<BM, kSmall, NW> rows;
   rows.scan(gd.seg_off, gd.n_expert, s_wave_sum);
-  constexpr int kF = kSmall ? narrow_factor<BM, BN, GEMM_DGRAD>() : 1;
+  constexpr int kF = kSmall ? narrow_factor<BM, BN, DMODE>() : 1;
   const bool narrow = kF > 1 && rows.rows_s * tiles_n_d <= kNarrowMax &&
                       gd.out_feat >= kNarrowMinK;
   const int cols_s = narrow ? tiles_n_d * kF : tiles_n_d;
@@ -1740,11 +1742,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_bwd_kernel(GemmArgs gd, Gem
   const TileRows where = rows.find(gd.seg_off, v, small, s_owner);
   if constexpr (kSmall) {
     if (small) {
-      remainder_tile<T, BM, BN, GEMM_DGRAD>(gd, smem, where, n_tile, narrow);
+      remainder_tile<T, BM, BN, DMODE>(gd, smem, where, n_tile, narrow);
       return;
     }
   }
-  edge_aware_tile<T, BM, BN, BK, WM, WN, NS, GEMM_DGRAD>(gd, smem, where, n_tile);
+  edge_aware_tile<T, BM, BN, BK, WM, WN, NS, DMODE>(gd, smem, where, n_tile);
 }
 
 // ------------------------------------------------------------------ host side
@@ -1757,7 +1759,7 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   constexpr size_t pipe_bytes = NS * (ATile::kBytes + BTile::kBytes);
   // staged output tile (+ the activation table of a fused DGRAD epilogue)
   constexpr size_t out_bytes =
-      MODE == GEMM_DGRAD ? (size_t)kActTabLdsOffset + kActTabBytes : (size_t)BM * (BN + 8) * 2;
+      MODE == GEMM_DGRAD_ACT ? (size_t)kActTabLdsOffset + kActTabBytes : (size_t)BM * (BN + 8) * 2;
   constexpr size_t small_bytes = has_small_tiles<BM, BN, MODE>()
       ? (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2 : 0;
   constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
@@ -1850,13 +1852,19 @@ static int launch_t(int mode, const GemmArgs& g, hipStream_t s) {
       FMOE_REQUIRE(g.act_out == nullptr, FMOE_ERR_UNSUPPORTED,
                    "grouped GEMM: the fused activation is a bf16 kernel");
       return launch_mode<T, GEMM_FWD>(g, s);
-    case GEMM_DGRAD: return launch_mode<T, GEMM_DGRAD>(g, s);
+    case GEMM_DGRAD:
+      if constexpr (std::is_same<T, __hip_bfloat16>::value) {
+        if (g.act_pre) return launch_mode<T, GEMM_DGRAD_ACT>(g, s);
+      }
+      FMOE_REQUIRE(g.act_pre == nullptr, FMOE_ERR_UNSUPPORTED,
+                   "grouped GEMM: the fused activation is a bf16 kernel");
+      return launch_mode<T, GEMM_DGRAD>(g, s);
     default: return launch_mode<T, GEMM_WGRAD>(g, s);
   }
 }
 
 // dX and dW of one linear in one launch of 256x256 tiles, K slices of BK in NS stages.
-template <typename T, int BK, int NS>
+template <typename T, int BK, int NS, bool ACT = false>
 static int launch_bwd_fused(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
   constexpr int BM = 256, BN = 256, WM = 2, WN = 2, NT = WM * WN * 64;
   constexpr size_t pipe_bytes = (size_t)NS * (BM + BN) * BK * 2;
@@ -1865,7 +1873,15 @@ static int launch_bwd_fused(const GemmArgs& gd, const GemmArgs& gw, hipStream_t 
   constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
   constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
-  auto kern = gemm_bwd_kernel<T, BM, BN, BK, WM, WN, NS>;
+  if (gd.act_pre) {
+    if constexpr (std::is_same<T, __hip_bfloat16>::value) {
+      if (!ACT) return launch_bwd_fused<T, BK, NS, true>(gd, gw, s);
+    } else {
+      FMOE_REQUIRE(false, FMOE_ERR_UNSUPPORTED,
+                   "grouped GEMM: the fused activation is a bf16 kernel");
+    }
+  }
+  auto kern = gemm_bwd_kernel<T, BM, BN, BK, WM, WN, NS, ACT>;
   FMOE_SET_DYNAMIC_LDS_ONCE(kern, lds_bytes);
   const int tiles_n_d = ceil_div(gd.in_feat, BN);
   const int tiles_n_w = ceil_div(gw.in_feat, BN), tiles_m_w = ceil_div(gw.out_feat, BM);
@@ -1893,7 +1909,7 @@ static int launch_bwd_t(const GemmArgs& gd, const GemmArgs& gw, hipStream_t s) {
   const int pd = pick_tile<GEMM_DGRAD>(gd), pw = pick_tile<GEMM_WGRAD>(gw);
   if (pd == 4 && pw == 4) return launch_bwd_fused<T, 64, 2>(gd, gw, s);  // forced
   if (pd != 1 || pw != 1) {
-    const int rc = launch_mode<T, GEMM_DGRAD>(gd, s);
+    const int rc = launch_t<T>(GEMM_DGRAD, gd, s);
     return rc ? rc : launch_mode<T, GEMM_WGRAD>(gw, s);
   }
   // K slices of 64 in two stages measured 2-3% faster than four stages of 32
