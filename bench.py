@@ -57,10 +57,12 @@ PEAK = {"hbm": 8.0e12, "bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 # whose traffic is known (FETCH_SIZE x 1.035 on cfg2 and cfg5, x 0.998 on cfg4;
 # WRITE_SIZE x 1.000).  Only the workloads that were measured have an entry.
 MEASURED_TRAFFIC = {
-    ("cfg2", "grouped_linear_bwd"): (310.4 + 213.1) * 2 ** 20,
-    ("cfg2", "grouped_linear_fwd"): (155.0 + 144.0) * 2 ** 20,
-    ("cfg4", "grouped_linear_bwd"): (5968.4 + 1507.1) * 2 ** 20,
-    ("cfg4", "grouped_linear_fwd"): (2921.7 + 1024.0) * 2 ** 20,
+    ("cfg2", "grouped_linear_bwd"): (311.1 + 214.6) * 2 ** 20,       # avg of both layers
+    ("cfg2", "grouped_linear_fwd"): (172.1 + 32.2) * 2 ** 20,
+    ("cfg2", "grouped_linear_fwd_act"): (138.7 + 257.0) * 2 ** 20,
+    ("cfg4", "grouped_linear_bwd"): (5962.0 + 1517.7) * 2 ** 20,     # avg of both layers
+    ("cfg4", "grouped_linear_fwd"): (2927.7 + 258.0) * 2 ** 20,
+    ("cfg4", "grouped_linear_fwd_act"): (2929.8 + 1799.0) * 2 ** 20,
     ("cfg5", "grouped_linear_bwd"): (1247.1 + 961.3) * 2 ** 20,
     ("cfg5", "grouped_linear_fwd"): (811.3 + 216.0) * 2 ** 20,
 }
