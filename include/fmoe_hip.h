@@ -257,8 +257,10 @@ int fmoe_grouped_linear_bwd(const void* dy, const void* x, const void* w,
  * the exact GELU of torch.nn.GELU().  Where the bf16 matrix-core kernel runs, both
  * leave the same output tiles (the activation kernel's own table of gelu(x) for
  * 16-bit x, applied to the rounded y: the same bits as fmoe_gelu_fwd over y); for
- * other dtypes and shapes the entry point runs that kernel behind the GEMM.  Rows of
- * y_act behind seg_off[n_expert] are left untouched, like those of y.
+ * other dtypes and shapes, and below about 768 rows per expert (where the separate
+ * kernel is as fast), the entry point runs that kernel behind the GEMM;
+ * FMOE_FUSE_FWD_ACT=0 in the environment makes it do so always (a tuning aid).  Rows
+ * of y_act behind seg_off[n_expert] are left untouched, like those of y.
  */
 int fmoe_grouped_linear_fwd_act(const void* x, const void* w, const void* bias,
                                 const int32_t* seg_off, void* y, void* y_act,
