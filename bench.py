@@ -261,9 +261,9 @@ def main():
                     help="workload; the default is the largest single-GPU configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--binding", default="ctypes", choices=["ctypes", "compiled"],
-                    help="Python binding of the C ABI: the ctypes module (default; carries the "
-                         "per-op event hooks the roofline figures come from) or the compiled "
-                         "pybind11 extension (whole-step timing and host enqueue time only)")
+                    help="Python binding of the C ABI: the ctypes module (default; needs "
+                         "nothing but the shared library) or the compiled pybind11 extension "
+                         "(less host time per step); both feed the per-op event hook")
     ap.add_argument("--graph", action="store_true",
                     help="also time the same steps replayed from one HIP graph (extra field)")
     args = ap.parse_args()
@@ -317,7 +317,7 @@ def main():
     # table, and which op takes the largest share of a step.  (Every event pair
     # idles the GPU for a few microseconds, so the timed region below keeps
     # them on that one op only.)
-    hooks = args.binding == "ctypes"
+    hooks = True    # both bindings feed the per-op event hook
     survey_steps = min(5, max(1, args.steps))
     records = []
     fmoe_cuda.profile_hook = lambda name, a, b: records.append((name, a, b))
@@ -356,8 +356,6 @@ def main():
     traffic = MEASURED_TRAFFIC.get((args.config, dom))
     roofline["traffic"] = None if traffic is None else round(traffic)
     roofline["avg_launch_us"] = kernels[dom]["avg_us"] if hooks else None
-    if not hooks:
-        roofline = None     # no per-op events on the compiled binding
 
     result = {
         "metric": "MoE-MLP fwd+bwd tokens/s @1 MI355X",
