@@ -30,11 +30,22 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.dirname(HERE))
+
+
+def _library_build():
+    """fastmoe_amd/build.py (the library's own compiler and flags), loaded by path: the
+    package itself is not imported, so no library has to exist yet."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location(
+        "fmoe_library_build", os.path.join(os.path.dirname(HERE), "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
 
 
 def compile_to_assembly(out_path: str, all_dtypes: bool) -> None:
-    import build as _build  # fastmoe_amd/build.py: the library's own compiler and flags
+    _build = _library_build()
 
     cmd = [_build.HIPCC, *_build.FLAGS, "--cuda-device-only", "-S",
            os.path.join(HERE, "gemm_mfma.hip"), "-o", out_path]

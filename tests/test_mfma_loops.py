@@ -12,11 +12,8 @@ from conftest import ROOT
 
 
 def test_compiler_leaves_the_mfma_loops_alone():
-    sys.path.insert(0, os.path.join(ROOT, "fastmoe_amd"))
-    try:
-        import build as lib_build
-    finally:
-        sys.path.pop(0)
+    from fastmoe_amd import build as lib_build
+
     if not os.path.exists(lib_build.HIPCC):
         pytest.skip("no hipcc on this machine")
     res = subprocess.run([sys.executable, os.path.join(ROOT, "fastmoe_amd", "csrc",
