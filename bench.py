@@ -121,14 +121,17 @@ class PresetGate(torch.nn.Module):
         return idx, score.to(self.dtype)
 
 
-def build_layer(cfg: dict, device="cuda"):
+def build_layer(cfg: dict, device="cuda", fused=True):
+    """The layer with seeded weights, its input and the gradient of its output.
+    fused=False builds the reference's expert layout, one module per expert
+    (fmoe/transformer.py:51-55), with values from the same generator."""
     from fastmoe_amd import FMoETransformerMLP
 
     dtype = DTYPES[cfg["dtype"]]
     PresetGate.cfg = cfg
     torch.manual_seed(0)
     layer = FMoETransformerMLP(num_expert=cfg["E"], d_model=cfg["d"], d_hidden=cfg["h"],
-                               top_k=cfg["k"], gate=PresetGate)
+                               top_k=cfg["k"], gate=PresetGate, fused=fused)
     g = torch.Generator().manual_seed(1)
     with torch.no_grad():
         for p in layer.experts.parameters():
@@ -252,6 +255,69 @@ def cpu_baseline(cfg: dict, layer, x, target_seconds: float = 15.0):
     }
 
 
+def yardstick(cfg: dict, layer, seg_off, iters: int = 5):
+    """The expert GEMMs of this workload as the BLAS library runs them: torch.mm
+    (hipBLASLt) on the same weights and row segments.  Two forms per product and layer:
+    `loop`, one call per expert on its own rows (the reference's algorithm,
+    cuda/parallel_linear.cuh:55-163, a loop of BLAS calls), and `dense`, ONE call with
+    all rows against one expert's weight (no ragged edges, no small problems: what
+    the library reaches on this shape at its best).  Untimed leg, for comparison only:
+    nothing of the product path runs through it."""
+    ex = layer.experts
+    dtype = DTYPES[cfg["dtype"]]
+    seg = seg_off.cpu().tolist()
+    n = seg[-1]
+    dev = ex.htoh4.weight.device
+    g = torch.Generator(device="cpu").manual_seed(7)
+    out = {"what": "torch.mm (hipBLASLt) on this workload's weights and row segments; "
+                   "loop = one call per expert (the reference's algorithm), dense = one call, "
+                   "all rows x one expert's weight", "products": {}}
+    peak = PEAK[cfg["dtype"]]
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        b.synchronize()
+        return a.elapsed_time(b) * 1e-3 / iters
+
+    for name, lin in (("layer1", ex.htoh4), ("layer2", ex.h4toh)):
+        w = lin.weight.detach()                       # [E, out, in]
+        out_f, in_f = w.shape[1], w.shape[2]
+        x = (torch.randn(n, in_f, generator=g) * 0.5).to(dtype).to(dev)
+        dy = (torch.randn(n, out_f, generator=g) * 0.5).to(dtype).to(dev)
+        live = [(e, seg[e], seg[e + 1]) for e in range(len(seg) - 1) if seg[e + 1] > seg[e]]
+        flop = 2.0 * n * in_f * out_f
+        forms = {
+            "fwd": (lambda: [torch.mm(x[a:b], w[e].t()) for e, a, b in live],
+                    lambda: torch.mm(x, w[0].t())),
+            "dgrad": (lambda: [torch.mm(dy[a:b], w[e]) for e, a, b in live],
+                      lambda: torch.mm(dy, w[0])),
+            "wgrad": (lambda: [torch.mm(dy[a:b].t(), x[a:b]) for e, a, b in live],
+                      lambda: torch.mm(dy.t(), x)),
+        }
+        for prod, (loop, dense) in forms.items():
+            t_loop, t_dense = timed(loop), timed(dense)
+            out["products"][f"{name}_{prod}"] = {
+                "loop_us": round(t_loop * 1e6, 1),
+                "loop_frac_of_peak": round(flop / t_loop / peak, 4),
+                "dense_us": round(t_dense * 1e6, 1),
+                "dense_frac_of_peak": round(flop / t_dense / peak, 4),
+            }
+        del x, dy
+    p = out["products"]
+    for form in ("loop", "dense"):
+        tot = sum(v[f"{form}_us"] for v in p.values())
+        out[f"{form}_total_us"] = round(tot, 1)
+        out[f"{form}_frac_of_peak"] = round(
+            12.0 * n * cfg["d"] * cfg["h"] / (tot * 1e-6) / peak, 4)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -260,10 +326,17 @@ def main():
     ap.add_argument("--config", default="cfg4", choices=sorted(CONFIGS),
                     help="workload; the default is the largest single-GPU configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--binding", default="ctypes", choices=["ctypes", "compiled"],
-                    help="Python binding of the C ABI: the ctypes module (default; needs "
-                         "nothing but the shared library) or the compiled pybind11 extension "
-                         "(less host time per step); both feed the per-op event hook")
+    ap.add_argument("--binding", default="compiled", choices=["compiled", "ctypes"],
+                    help="Python binding of the C ABI: the compiled pybind11 extension "
+                         "(default) or the ctypes calls (need nothing but the shared "
+                         "library, more host time per step); both feed the per-op event hook")
+    ap.add_argument("--layout", default="fused", choices=["fused", "list"],
+                    help="expert parameters as [E, out, in] tensors (default) or as the "
+                         "reference's list of single-expert modules (the kernels then read "
+                         "the weights through pointer tables); list implies --no-cpu "
+                         "--no-yardstick")
+    ap.add_argument("--no-yardstick", action="store_true",
+                    help="skip the untimed torch.mm (hipBLASLt) comparison of the expert GEMMs")
     ap.add_argument("--graph", action="store_true",
                     help="also time the same steps replayed from one HIP graph (extra field)")
     args = ap.parse_args()
@@ -273,13 +346,14 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (there is no CPU fallback of the hot path)")
 
-    if args.binding == "compiled":
-        os.environ["FMOE_BINDING"] = "compiled"
+    os.environ["FMOE_BINDING"] = args.binding
     from fastmoe_amd import fmoe_cuda
 
     assert fmoe_cuda.BINDING == args.binding
     cfg = dict(CONFIGS[args.config], name=args.config)
-    layer, x, dy = build_layer(cfg)
+    if args.layout == "list":
+        args.no_cpu = args.no_yardstick = True
+    layer, x, dy = build_layer(cfg, fused=args.layout == "fused")
     x.requires_grad_(True)
 
     for _ in range(args.warmup):
@@ -372,6 +446,7 @@ def main():
         "dtype": cfg["dtype"],
         "data": "synthetic",
         "binding": args.binding,
+        "expert_layout": args.layout,
         "config": {
             "workload": (f"{args.config}: {cfg['T']} tokens, d_model {cfg['d']}, d_hidden "
                          f"{cfg['h']}, {cfg['E']} experts, top-{cfg['k']}, {cfg['dtype']}; "
@@ -385,6 +460,18 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    # the step's own GEMMs next to the library's, same shapes: the four grouped launches
+    gemm_us = sum(kernels[k]["total_ms_per_step"] * 1e3 for k in kernels
+                  if k.startswith("grouped_linear"))
+    result["gemm_frac_of_peak_step"] = round(
+        12.0 * n_valid * cfg["d"] * cfg["h"] / (gemm_us * 1e-6) / PEAK[cfg["dtype"]], 4) \
+        if gemm_us > 0 else None
+    if not args.no_yardstick:
+        from fastmoe_amd.functions import RoutePlan
+
+        with torch.no_grad():
+            plan = RoutePlan(idx, cfg["E"])
+        result["yardstick"] = yardstick(cfg, layer, plan.segments.seg_off)
     if args.graph:
         result["hip_graph"] = graph_replay(layer, x, dy, cfg, args.steps)
     if not args.no_cpu:

@@ -11,11 +11,11 @@ from .linear import FMoELinear
 from .transformer import FMoETransformerMLP
 
 
-def install_as_fmoe_cuda(compiled: bool = False) -> None:
-    """Registers the operator module as `fmoe_cuda`, so that the reference's
+def install_as_fmoe_cuda(compiled: bool = True) -> None:
+    """Registers an operator module as `fmoe_cuda`, so that the reference's
     own Python package (`import fmoe_cuda` in fmoe/functions.py:9) binds to the
-    MI355X kernels: the ctypes module, or with `compiled=True` the pybind11
-    extension of that name (cuda/fmoe_cuda.cpp:104-125 rebuilt on the C ABI)."""
+    MI355X kernels: the pybind11 extension of that name (cuda/fmoe_cuda.cpp:104-125
+    rebuilt on the C ABI), or with `compiled=False` the ctypes module."""
     import sys
 
     if compiled:
@@ -23,7 +23,7 @@ def install_as_fmoe_cuda(compiled: bool = False) -> None:
 
         sys.modules["fmoe_cuda"] = _ext.load()
     else:
-        sys.modules.setdefault("fmoe_cuda", fmoe_cuda)
+        sys.modules["fmoe_cuda"] = fmoe_cuda.ctypes_ops
 
 
 __all__ = ["FMoE", "FMoELinear", "FMoETransformerMLP", "BaseGate", "NaiveGate",

@@ -21,11 +21,12 @@ def load(build_if_missing: bool = True):
 
     _lib.load()                      # libfmoe_hip.so first: the extension links to it
     path = _build.ext_path()
+    # a binary compiled from another state of its source or of the C ABI header
     stale = (os.path.exists(path) and os.path.exists(_build.EXT_SRC)
-             and os.path.getmtime(path) < os.path.getmtime(_build.EXT_SRC))
+             and _build.ext_built_hash(path) != _build.ext_source_hash())
     if not os.path.exists(path) or stale:
         if not build_if_missing:
-            raise ImportError(f"{path} is missing or older than its source; run "
+            raise ImportError(f"{path} is missing or was built from other sources; run "
                               "`python fastmoe_amd/build.py`")
         _build.build_extension(verbose=False)
     import torch  # noqa: F401  (the module links to libtorch)

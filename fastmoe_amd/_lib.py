@@ -18,6 +18,7 @@ _lib = None
 SIGNATURES = {
     "fmoe_version": (c_char_p, []),
     "fmoe_last_error": (c_char_p, []),
+    "fmoe_init": (c_int, [c_void_p]),
     "fmoe_expert_count": (c_int, [c_void_p, c_int64, c_void_p, c_int32, c_void_p]),
     "fmoe_route_workspace_bytes": (c_int64, [c_int64, c_int32]),
     "fmoe_assign_pos": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int32,
@@ -54,6 +55,13 @@ SIGNATURES = {
     "fmoe_grouped_linear_bwd_act": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_void_p, c_int64,
                                             c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "fmoe_grouped_linear_fwd_ptrs": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                             c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                             c_int, c_void_p]),
+    "fmoe_grouped_linear_bwd_ptrs": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                             c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                             c_int64, c_int64, c_int, c_void_p]),
+    "fmoe_pointer_table": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "fmoe_seg_off_from_host_counts": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "fmoe_topk_softmax_fwd": (c_int, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p,
                                       c_int, c_void_p]),

@@ -18,9 +18,11 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfmoe_hip.so")
 
-SOURCES = ["api.hip", "route.hip", "dispatch.hip", "gate.hip", "act.hip", "gemm_simt.hip", "gemm_mfma.hip",
-           "gemm_mfma_wide.hip"]
-HEADERS = ["common.h", "gemm.h", "dma_desc.h", os.path.join("..", "..", "include", "fmoe_hip.h")]
+# the two heavy translation units first, so that they compile side by side
+SOURCES = ["gemm_mfma_bf16.hip", "gemm_mfma_f16.hip", "api.hip", "route.hip", "dispatch.hip",
+           "gate.hip", "act.hip", "gemm_simt.hip", "gemm_mfma.hip", "gemm_mfma_wide.hip"]
+HEADERS = ["common.h", "gemm.h", "dma_desc.h", "gemm_mfma_impl.h",
+           os.path.join("..", "..", "include", "fmoe_hip.h")]
 # the library carries a digest of the files it was built from behind this marker
 HASH_MARKER = "fmoe-src:"
 
@@ -98,6 +100,31 @@ EXT_DIR = os.path.join(PKG_DIR, "ext")
 EXT_SRC = os.path.join(CSRC, "fmoe_cuda_ext.cpp")
 
 
+EXT_HASH_MARKER = "fmoe-ext:"
+
+
+def ext_source_hash() -> str:
+    """Digest of what the extension is compiled from: its source and the C ABI header."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for path in (EXT_SRC, os.path.join(PKG_DIR, "..", "include", "fmoe_hip.h")):
+        with open(path, "rb") as f:
+            h.update(f.read() + b"\0")
+    return h.hexdigest()[:12]
+
+
+def ext_built_hash(path: str):
+    """The digest a built extension carries (None if it has none)."""
+    with open(path, "rb") as f:
+        blob = f.read()
+    at = blob.find(EXT_HASH_MARKER.encode())
+    if at < 0:
+        return None
+    at += len(EXT_HASH_MARKER)
+    return blob[at:at + 12].decode("ascii", "replace")
+
+
 def ext_path() -> str:
     import sysconfig
 
@@ -118,6 +145,7 @@ def build_extension(verbose: bool = True) -> str:
     torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
     cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
            "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=fmoe_cuda",
+           f'-DFMOE_EXT_SOURCE_HASH="{ext_source_hash()}"',
            f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
            "-Wno-deprecated-declarations"]
     cmd += ["-I" + p for p in ce.include_paths("cuda")]

@@ -4,18 +4,18 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <algorithm>
+
 #include "gemm.h"
 
 namespace fmoe {
 
 static thread_local char g_err[512] = "";
-static int g_gemm_path = 0;  // 0 = automatic, 1 = scalar kernel only (2..5 set g_tile instead)
-// tuning aid: FMOE_GEMM_TILE=1..4 forces one MFMA tile configuration (0 / unset = automatic)
-static const int g_env_tile = getenv("FMOE_GEMM_TILE") ? atoi(getenv("FMOE_GEMM_TILE")) : 0;
-static int g_tile = g_env_tile;
-// tuning aid: FMOE_FUSE_FWD_ACT=0 keeps the forward activation a kernel of its own
-static const bool g_fuse_fwd_act =
-    !(getenv("FMOE_FUSE_FWD_ACT") && atoi(getenv("FMOE_FUSE_FWD_ACT")) == 0);
+// What fmoe_set_gemm_path() selected, per calling thread (a testing aid; every
+// thread starts with the automatic choice).
+static thread_local int g_gemm_path = 0;   // 0 = automatic, 1 = scalar kernel only
+static thread_local int g_tile = 0;        // 1..4 = one MFMA tile configuration forced
+static thread_local bool g_fuse_fwd_act = true;  // false: the forward activation stays a kernel
 
 int set_error(int code, const char* fmt, ...) {
   va_list ap;
@@ -138,11 +138,26 @@ extern "C" const char* fmoe_version(void) {
 }
 extern "C" const char* fmoe_last_error(void) { return g_err; }
 
+// One-time set-up of the current GPU, all of which the entry points otherwise do
+// at their first call: the address of fmoe_route_static's built-in buffer and the
+// activation tables of the 16-bit kernels (built on `stream`, waited for).
+extern "C" int fmoe_init(void* stream) {
+  int rc = route_static_init();
+  if (rc) return rc;
+  const uint16_t* fwd = nullptr;
+  const float* bwd = nullptr;
+  rc = gelu_fwd_table(FMOE_BF16, (hipStream_t)stream, &fwd);
+  if (rc) return rc;
+  return gelu_bwd_table(FMOE_BF16, (hipStream_t)stream, &bwd);
+}
+
 extern "C" int fmoe_set_gemm_path(int path) {
-  FMOE_REQUIRE(path >= 0 && path <= 5, FMOE_ERR_INVALID, "gemm path must be 0..5");
-  // 2..5: matrix-core kernel with tile configuration 1..4 forced (tests, tuning)
+  FMOE_REQUIRE(path >= 0 && path <= 6, FMOE_ERR_INVALID, "gemm path must be 0..6");
+  // 2..5: matrix-core kernel with tile configuration 1..4 forced; 6: automatic, but
+  // the forward activation runs as a kernel of its own behind the GEMM
   g_gemm_path = path == 1 ? 1 : 0;
-  g_tile = path >= 2 ? path - 1 : g_env_tile;
+  g_tile = path >= 2 && path <= 5 ? path - 1 : 0;
+  g_fuse_fwd_act = path != 6;
   return FMOE_OK;
 }
 
@@ -178,34 +193,24 @@ extern "C" int fmoe_seg_off_from_host_counts(const int64_t* expert_count_host,
   return FMOE_OK;
 }
 
-extern "C" int fmoe_grouped_linear_fwd(const void* x, const void* w,
-                                       const void* bias, const int32_t* seg_off,
-                                       void* y, int64_t n_rows, int64_t in_feat,
-                                       int64_t out_feat, int64_t n_expert,
-                                       int dtype, void* stream) {
-  int rc = check_linear("grouped_linear_fwd", n_rows, in_feat, out_feat, n_expert, dtype);
+// Forward of the grouped linear layer, with the weights (and the bias) as one
+// [E, ...] array or as tables of per-expert pointers, and optionally the activation
+// behind it: y_act = gelu(y) from the same tiles where the bf16 matrix-core kernel
+// runs, by the activation kernel over y otherwise.
+static int linear_fwd(const char* who, const void* x, const void* w, const void* const* w_table,
+                      const void* bias, const void* const* bias_table, const int32_t* seg_off,
+                      void* y, void* y_act, bool want_act, int64_t n_rows, int64_t in_feat,
+                      int64_t out_feat, int64_t n_expert, int dtype, void* stream) {
+  int rc = check_linear(who, n_rows, in_feat, out_feat, n_expert, dtype);
   if (rc) return rc;
   if (n_rows == 0) return FMOE_OK;
-  FMOE_REQUIRE(x && w && seg_off && y, FMOE_ERR_INVALID,
-               "grouped_linear_fwd: null pointer");
-  GemmArgs g{x, w, y, bias, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
-  return run_gemm(GEMM_FWD, g, dtype, (hipStream_t)stream);
-}
-
-// Forward of the grouped linear layer with the activation behind it: y as
-// fmoe_grouped_linear_fwd writes it and y_act = gelu(y), from the same tiles where
-// the bf16 matrix-core kernel runs, by the activation kernel over y otherwise.
-extern "C" int fmoe_grouped_linear_fwd_act(const void* x, const void* w, const void* bias,
-                                           const int32_t* seg_off, void* y, void* y_act,
-                                           int64_t n_rows, int64_t in_feat, int64_t out_feat,
-                                           int64_t n_expert, int dtype, void* stream) {
-  int rc = check_linear("grouped_linear_fwd_act", n_rows, in_feat, out_feat, n_expert, dtype);
-  if (rc) return rc;
-  if (n_rows == 0) return FMOE_OK;
-  FMOE_REQUIRE(x && w && seg_off && y && y_act, FMOE_ERR_INVALID,
-               "grouped_linear_fwd_act: null pointer");
+  FMOE_REQUIRE(x && (w || w_table) && seg_off && y && (y_act || !want_act), FMOE_ERR_INVALID,
+               "%s: null pointer", who);
   hipStream_t s = (hipStream_t)stream;
   GemmArgs g{x, w, y, bias, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
+  g.w_table = w_table;
+  g.bias_table = bias_table;
+  if (!want_act) return run_gemm(GEMM_FWD, g, dtype, s);
   // Worth it from about 768 rows per expert on (measured: 12 % of GEMM + activation
   // kernel at 1024 rows per expert, 5 % at 4096, level at 512, where half of the tiles
   // are remainder tiles that pay the table and the second store for few rows); a
@@ -224,10 +229,60 @@ extern "C" int fmoe_grouped_linear_fwd_act(const void* x, const void* w, const v
   return fmoe_gelu_fwd(y, y_act, n_rows * out_feat, seg_off + n_expert, out_feat, dtype, stream);
 }
 
+extern "C" int fmoe_grouped_linear_fwd(const void* x, const void* w,
+                                       const void* bias, const int32_t* seg_off,
+                                       void* y, int64_t n_rows, int64_t in_feat,
+                                       int64_t out_feat, int64_t n_expert,
+                                       int dtype, void* stream) {
+  return linear_fwd("grouped_linear_fwd", x, w, nullptr, bias, nullptr, seg_off, y, nullptr,
+                    false, n_rows, in_feat, out_feat, n_expert, dtype, stream);
+}
+
+extern "C" int fmoe_grouped_linear_fwd_act(const void* x, const void* w, const void* bias,
+                                           const int32_t* seg_off, void* y, void* y_act,
+                                           int64_t n_rows, int64_t in_feat, int64_t out_feat,
+                                           int64_t n_expert, int dtype, void* stream) {
+  return linear_fwd("grouped_linear_fwd_act", x, w, nullptr, bias, nullptr, seg_off, y, y_act,
+                    true, n_rows, in_feat, out_feat, n_expert, dtype, stream);
+}
+
+extern "C" int fmoe_grouped_linear_fwd_ptrs(const void* x, const void* const* w_ptrs,
+                                            const void* const* bias_ptrs,
+                                            const int32_t* seg_off, void* y, void* y_act,
+                                            int64_t n_rows, int64_t in_feat, int64_t out_feat,
+                                            int64_t n_expert, int dtype, void* stream) {
+  return linear_fwd("grouped_linear_fwd_ptrs", x, nullptr, w_ptrs, nullptr, bias_ptrs, seg_off, y,
+                    y_act, y_act != nullptr, n_rows, in_feat, out_feat, n_expert, dtype, stream);
+}
+
+// A device array of pointers from a host array, written by a small kernel that
+// carries the values as its arguments: no staging copy, nothing to keep alive, no
+// host synchronisation.
+struct PtrChunk { const void* v[256]; };
+__global__ void write_pointers_kernel(PtrChunk c, const void** dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = c.v[i];
+}
+
+extern "C" int fmoe_pointer_table(const void* const* host_ptrs, int64_t n, const void** table,
+                                  void* stream) {
+  FMOE_REQUIRE(host_ptrs && table && n >= 1, FMOE_ERR_INVALID, "pointer_table: bad arguments");
+  hipStream_t s = (hipStream_t)stream;
+  for (int64_t done = 0; done < n; done += 256) {
+    PtrChunk chunk;
+    const int fill = (int)std::min<int64_t>(256, n - done);
+    for (int i = 0; i < fill; ++i) chunk.v[i] = host_ptrs[done + i];
+    hipLaunchKernelGGL(write_pointers_kernel, dim3(1), dim3(256), 0, s, chunk, table + done, fill);
+    FMOE_LAUNCH_CHECK("write_pointers");
+  }
+  return FMOE_OK;
+}
+
 // Backward of the grouped linear layer; with act_pre, dx is further multiplied
 // by gelu'(act_pre): inside the DGRAD tiles' epilogue where the bf16 matrix-core
 // kernel runs, by the activation kernel over dx otherwise.
-static int linear_bwd(const void* dy, const void* x, const void* w, const int32_t* seg_off,
+static int linear_bwd(const void* dy, const void* x, const void* w, const void* const* w_table,
+                      const int32_t* seg_off,
                       const void* act_pre, void* dx, void* dw, void* dbias, int64_t n_rows,
                       int64_t in_feat, int64_t out_feat, int64_t n_expert, int dtype,
                       void* stream) {
@@ -248,6 +303,7 @@ static int linear_bwd(const void* dy, const void* x, const void* w, const int32_
     dbias = nullptr;  // comes out of the dW launch
   }
   GemmArgs gd{dy, w, dx, nullptr, seg_off, n_rows, (int)in_feat, (int)out_feat, (int)n_expert, g_tile};
+  gd.w_table = w_table;
   void* const dx_out = dx;
   const bool act_fused = act_pre && dx && n_rows > 0 && dtype == FMOE_BF16 && g_gemm_path == 0 &&
                          (uintptr_t)act_pre % 16 == 0 && gemm_mfma_supported(GEMM_DGRAD, gd, dtype);
@@ -257,7 +313,7 @@ static int linear_bwd(const void* dy, const void* x, const void* w, const int32_
     gd.act_pre = act_pre;
   }
   if (dx && dw && n_rows > 0 && g_gemm_path == 0) {
-    FMOE_REQUIRE(w != nullptr && x != nullptr, FMOE_ERR_INVALID,
+    FMOE_REQUIRE((w != nullptr || w_table != nullptr) && x != nullptr, FMOE_ERR_INVALID,
                  "grouped_linear_bwd: w or x is null");
     if (gemm_mfma_supported(GEMM_DGRAD, gd, dtype) && mfma_w) {
       rc = launch_gemm_mfma_bwd(gd, gw, dtype, s);
@@ -267,7 +323,8 @@ static int linear_bwd(const void* dy, const void* x, const void* w, const int32_
     }
   }
   if (dx && n_rows > 0) {
-    FMOE_REQUIRE(w != nullptr, FMOE_ERR_INVALID, "grouped_linear_bwd: w is null");
+    FMOE_REQUIRE(w != nullptr || w_table != nullptr, FMOE_ERR_INVALID,
+                 "grouped_linear_bwd: w is null");
     rc = run_gemm(GEMM_DGRAD, gd, dtype, s);
     if (rc) return rc;
   }
@@ -300,8 +357,8 @@ extern "C" int fmoe_grouped_linear_bwd(const void* dy, const void* x,
                                        int64_t n_rows, int64_t in_feat,
                                        int64_t out_feat, int64_t n_expert,
                                        int dtype, void* stream) {
-  return linear_bwd(dy, x, w, seg_off, nullptr, dx, dw, dbias, n_rows, in_feat, out_feat,
-                    n_expert, dtype, stream);
+  return linear_bwd(dy, x, w, nullptr, seg_off, nullptr, dx, dw, dbias, n_rows, in_feat,
+                    out_feat, n_expert, dtype, stream);
 }
 
 extern "C" int fmoe_grouped_linear_bwd_act(const void* dy, const void* x,
@@ -312,6 +369,18 @@ extern "C" int fmoe_grouped_linear_bwd_act(const void* dy, const void* x,
                                            int dtype, void* stream) {
   FMOE_REQUIRE(act_pre != nullptr || n_rows == 0 || dx == nullptr, FMOE_ERR_INVALID,
                "grouped_linear_bwd_act: act_pre is null");
-  return linear_bwd(dy, x, w, seg_off, act_pre, dx, dw, dbias, n_rows, in_feat, out_feat,
-                    n_expert, dtype, stream);
+  return linear_bwd(dy, x, w, nullptr, seg_off, act_pre, dx, dw, dbias, n_rows, in_feat,
+                    out_feat, n_expert, dtype, stream);
+}
+
+extern "C" int fmoe_grouped_linear_bwd_ptrs(const void* dy, const void* x,
+                                            const void* const* w_ptrs, const int32_t* seg_off,
+                                            const void* act_pre, void* dx, void* dw,
+                                            void* dbias, int64_t n_rows, int64_t in_feat,
+                                            int64_t out_feat, int64_t n_expert,
+                                            int dtype, void* stream) {
+  FMOE_REQUIRE(w_ptrs != nullptr || dx == nullptr || n_rows == 0, FMOE_ERR_INVALID,
+               "grouped_linear_bwd_ptrs: w_ptrs is null");
+  return linear_bwd(dy, x, nullptr, w_ptrs, seg_off, act_pre, dx, dw, dbias, n_rows, in_feat,
+                    out_feat, n_expert, dtype, stream);
 }

@@ -17,6 +17,9 @@ constexpr int kWave = 64;  // CDNA wavefront width
 // Records the text returned by fmoe_last_error() and hands back `code`.
 int set_error(int code, const char* fmt, ...);
 
+// Per-GPU set-up of fmoe_route_static (route.hip), part of fmoe_init().
+int route_static_init();
+
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
 #define FMOE_REQUIRE(cond, code, ...)                 \

@@ -10,8 +10,13 @@
 #include <c10/hip/HIPStream.h>
 #include <c10/core/DeviceGuard.h>
 
+#include <hip/hip_runtime_api.h>
+
+#include <map>
+#include <mutex>
 #include <string>
 #include <tuple>
+#include <utility>
 #include <vector>
 
 #include "../../include/fmoe_hip.h"
@@ -57,10 +62,28 @@ void* stream_of(const Tensor& t) {
 
 void* ptr(const OptTensor& t) { return t.has_value() && t->defined() ? t->data_ptr() : nullptr; }
 
+// Routing workspace for a call on torch's current stream of `like`'s device.  One
+// buffer per (device, stream) is kept and reused: launches on one stream run in
+// order, and nothing in the workspace outlives a call.  A stream under graph capture
+// gets a fresh tensor instead, which then belongs to the graph's own memory pool.
 Tensor workspace(int64_t numel, int64_t n_expert, const Tensor& like) {
-  const int64_t bytes = fmoe_route_workspace_bytes(numel, (int32_t)n_expert);
+  int64_t bytes = fmoe_route_workspace_bytes(numel, (int32_t)n_expert);
   need(bytes >= 0, "route workspace: bad sizes");
-  return torch::empty({bytes > 0 ? bytes : 1}, like.options().dtype(at::kByte));
+  if (bytes < 1) bytes = 1;
+  auto opts = like.options().dtype(at::kByte);
+  void* stream = stream_of(like);
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing((hipStream_t)stream, &capturing) != hipSuccess ||
+      capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return torch::empty({bytes}, opts);
+  }
+  static std::mutex mu;
+  static std::map<std::pair<int, void*>, Tensor> cache;
+  std::lock_guard<std::mutex> lock(mu);
+  Tensor& ws = cache[{(int)like.device().index(), stream}];
+  if (!ws.defined() || ws.numel() < bytes) ws = torch::empty({std::max<int64_t>(bytes, 1 << 16)}, opts);
+  return ws;
 }
 
 // ---------------------------------------------------------------- reference surface
@@ -86,10 +109,22 @@ void assign_pos(Tensor cum_count, Tensor gate, Tensor pos) {
 }
 
 // seg_off (device int32[E+1]) from the reference's host int64 counts, or from
-// device counts without a host round trip
-Tensor seg_off_from_counts(const Tensor& expert_count, const Tensor& like) {
+// device counts without a host round trip.  With host counts and rows >= 0 the
+// counts must not claim more rows than the buffers hold (the grouped kernels trust
+// seg_off); the reference assumes the sum equals the row count.
+Tensor seg_off_from_counts(const Tensor& expert_count, const Tensor& like, int64_t rows = -1) {
   need(expert_count.scalar_type() == at::kLong, "expert_count must be int64");
   const int64_t e = expert_count.numel();
+  if (!expert_count.is_cuda() && rows >= 0) {
+    const Tensor c = expert_count.contiguous();
+    int64_t total = 0;
+    for (int64_t i = 0; i < e; ++i) {
+      need(c.data_ptr<int64_t>()[i] >= 0, "expert_count holds a negative count");
+      total += c.data_ptr<int64_t>()[i];
+    }
+    need(total <= rows, "expert_count sums to " + std::to_string(total) + " rows, the buffer has " +
+                            std::to_string(rows));
+  }
   auto opts = like.options().dtype(at::kInt);
   if (expert_count.is_cuda()) {
     Tensor seg = torch::zeros({e + 1}, opts);
@@ -158,6 +193,7 @@ std::tuple<OptTensor, OptTensor, OptTensor> grouped_linear_bwd(Tensor dy, Tensor
   dev(x, "x", dy.scalar_type());
   dev(weight, "weight", dy.scalar_type());
   dev(seg_off, "seg_off", at::kInt);
+  need(x.dim() == 2 && weight.dim() == 3, "x must be 2-d and weight 3-d");
   const int64_t e = weight.size(0), out_f = weight.size(1), in_f = weight.size(2);
   const int64_t n = x.size(0);
   need(dy.dim() == 2 && dy.size(0) == n && dy.size(1) == out_f, "dy must be [rows, out]");
@@ -185,10 +221,90 @@ std::tuple<OptTensor, OptTensor, OptTensor> grouped_linear_bwd(Tensor dy, Tensor
   return {dx, dw, db};
 }
 
+// Device int64[n] of the tensors' data pointers (see fmoe_pointer_table)
+Tensor pointer_table(std::vector<Tensor> tensors) {
+  need(!tensors.empty(), "pointer_table: no tensors");
+  const Tensor& first = tensors[0];
+  std::vector<const void*> ptrs;
+  ptrs.reserve(tensors.size());
+  for (const Tensor& t : tensors) {
+    dev(t, "pointer_table entry", first.scalar_type());
+    need(t.device() == first.device() && t.sizes() == first.sizes(),
+         "pointer_table: tensors must share device and shape");
+    need((uintptr_t)t.data_ptr() % 16 == 0, "pointer_table: tensors must be 16-byte aligned");
+    ptrs.push_back(t.data_ptr());
+  }
+  c10::DeviceGuard guard(first.device());
+  Tensor table = torch::empty({(int64_t)ptrs.size()}, first.options().dtype(at::kLong));
+  check(fmoe_pointer_table(ptrs.data(), (int64_t)ptrs.size(), (const void**)table.data_ptr(),
+                           stream_of(first)),
+        "pointer_table");
+  return table;
+}
+
+py::object grouped_linear_fwd_ptrs(Tensor x, Tensor seg_off, Tensor w_table, OptTensor b_table,
+                                   int64_t out_f, bool with_gelu) {
+  dev(x, "x");
+  dev(seg_off, "seg_off", at::kInt);
+  dev(w_table, "w_table", at::kLong);
+  need(x.dim() == 2, "x must be [rows, in]");
+  const int64_t e = w_table.numel();
+  need(seg_off.numel() == e + 1, "seg_off must have E+1 entries");
+  if (b_table.has_value() && b_table->defined()) {
+    dev(*b_table, "b_table", at::kLong);
+    need(b_table->numel() == e, "b_table must have E entries");
+  }
+  c10::DeviceGuard guard(x.device());
+  Tensor y = torch::empty({x.size(0), out_f}, x.options());
+  OptTensor y_act;
+  if (with_gelu) y_act = torch::empty_like(y);
+  check(fmoe_grouped_linear_fwd_ptrs(x.data_ptr(), (const void* const*)w_table.data_ptr(),
+                                     (const void* const*)ptr(b_table), seg_off.data_ptr<int32_t>(),
+                                     y.data_ptr(), ptr(y_act), x.size(0), x.size(1), out_f, e,
+                                     dt(x, "x"), stream_of(x)),
+        "grouped_linear_fwd_ptrs");
+  if (with_gelu) return py::make_tuple(y, *y_act);
+  return py::cast(y);
+}
+
+std::tuple<OptTensor, OptTensor, OptTensor> grouped_linear_bwd_ptrs(
+    Tensor dy, Tensor x, Tensor seg_off, Tensor w_table, bool need_bias, bool need_dx,
+    bool need_dw, OptTensor act_pre) {
+  dev(dy, "dy");
+  dev(x, "x", dy.scalar_type());
+  dev(seg_off, "seg_off", at::kInt);
+  dev(w_table, "w_table", at::kLong);
+  need(x.dim() == 2 && dy.dim() == 2 && dy.size(0) == x.size(0),
+       "dy must be [rows, out] and x [rows, in]");
+  const int64_t e = w_table.numel(), n = x.size(0), in_f = x.size(1), out_f = dy.size(1);
+  need(seg_off.numel() == e + 1, "seg_off must have E+1 entries");
+  c10::DeviceGuard guard(dy.device());
+  OptTensor dx, dw, db;
+  if (need_dx) dx = torch::empty({n, in_f}, dy.options());
+  if (need_dw) dw = torch::empty({e, out_f, in_f}, dy.options());
+  if (need_bias) db = torch::empty({e, out_f}, dy.options());
+  const bool with_act = act_pre.has_value() && act_pre->defined() && need_dx;
+  if (with_act) {
+    dev(*act_pre, "act_pre", dy.scalar_type());
+    need(act_pre->dim() == 2 && act_pre->size(0) == n && act_pre->size(1) == in_f,
+         "act_pre must be [rows, in]");
+  }
+  if (need_dx || need_dw || need_bias)
+    check(fmoe_grouped_linear_bwd_ptrs(dy.data_ptr(), x.data_ptr(),
+                                       (const void* const*)w_table.data_ptr(),
+                                       seg_off.data_ptr<int32_t>(),
+                                       with_act ? act_pre->data_ptr() : nullptr, ptr(dx), ptr(dw),
+                                       ptr(db), n, in_f, out_f, e, dt(dy, "dy"), stream_of(dy)),
+          "grouped_linear_bwd_ptrs");
+  return {dx, dw, db};
+}
+
 Tensor linear_forward(Tensor input_buf, Tensor expert_count, Tensor weight, OptTensor bias) {
   dev(input_buf, "input_buf");
   c10::DeviceGuard guard(input_buf.device());
-  return grouped_linear_fwd(input_buf, seg_off_from_counts(expert_count, input_buf), weight, bias);
+  need(input_buf.dim() == 2, "input_buf must be [rows, in]");
+  return grouped_linear_fwd(input_buf, seg_off_from_counts(expert_count, input_buf, input_buf.size(0)),
+                            weight, bias);
 }
 
 std::vector<Tensor> linear_backward(Tensor grad_output_buf, Tensor input_buf, Tensor expert_count,
@@ -196,7 +312,9 @@ std::vector<Tensor> linear_backward(Tensor grad_output_buf, Tensor input_buf, Te
   dev(grad_output_buf, "grad_output_buf");
   dev(input_buf, "input_buf", grad_output_buf.scalar_type());
   c10::DeviceGuard guard(input_buf.device());
-  auto r = grouped_linear_bwd(grad_output_buf, input_buf, seg_off_from_counts(expert_count, input_buf),
+  need(input_buf.dim() == 2, "input_buf must be [rows, in]");
+  auto r = grouped_linear_bwd(grad_output_buf, input_buf,
+                              seg_off_from_counts(expert_count, input_buf, input_buf.size(0)),
                               weight, true, true, true, c10::nullopt);
   return {*std::get<0>(r), *std::get<1>(r), *std::get<2>(r)};
 }
@@ -442,6 +560,13 @@ PYBIND11_MODULE(fmoe_cuda, m) {
   m.def("grouped_linear_bwd", &grouped_linear_bwd, py::arg("dy"), py::arg("x"), py::arg("seg_off"),
         py::arg("weight"), py::arg("need_bias") = true, py::arg("need_dx") = true,
         py::arg("need_dw") = true, py::arg("act_pre") = py::none());
+  m.def("pointer_table", &pointer_table);
+  m.def("grouped_linear_fwd_ptrs", &grouped_linear_fwd_ptrs, py::arg("x"), py::arg("seg_off"),
+        py::arg("w_table"), py::arg("b_table"), py::arg("out_feat"),
+        py::arg("with_gelu") = false);
+  m.def("grouped_linear_bwd_ptrs", &grouped_linear_bwd_ptrs, py::arg("dy"), py::arg("x"),
+        py::arg("seg_off"), py::arg("w_table"), py::arg("need_bias") = true,
+        py::arg("need_dx") = true, py::arg("need_dw") = true, py::arg("act_pre") = py::none());
   m.def("gather_combine_fwd", &gather_combine_fwd);
   m.def("gather_combine_bwd", &gather_combine_bwd);
   m.def("scatter_reduce", &scatter_reduce);
@@ -460,4 +585,9 @@ PYBIND11_MODULE(fmoe_cuda, m) {
         });
   m.attr("MAX_GATE_TOP_K") = FMOE_MAX_GATE_TOP_K;
   m.attr("binding") = "compiled";
+#ifdef FMOE_EXT_SOURCE_HASH
+  // digest of this file and of the C ABI header it was compiled against: the loader
+  // rebuilds a binary whose digest differs from the sources beside it
+  m.attr("source_hash") = "fmoe-ext:" FMOE_EXT_SOURCE_HASH;
+#endif
 }

@@ -41,7 +41,39 @@ struct GemmArgs {
   // by 16-bit pattern of x (gelu_fwd_table()).
   void* act_out = nullptr;
   const uint16_t* act_fwd_table = nullptr;
+  // Experts whose parameters are separate allocations (the reference keeps one module
+  // per expert, fmoe/transformer.py:51-55, and its GEMM loop takes per-expert pointers,
+  // cuda/parallel_linear.cuh:69-87): DEVICE arrays of n_expert device pointers.  When
+  // w_table is not null, expert e's weight in FWD and DGRAD is w_table[e]
+  // ([out_feat, in_feat]) instead of b + e * out_feat * in_feat; when bias_table is
+  // not null, its forward bias is bias_table[e] ([out_feat]) instead of bias + e * out_feat.
+  const void* const* w_table = nullptr;
+  const void* const* bias_table = nullptr;
 };
+
+// Expert e's part of a per-expert operand: from the pointer table when there is one,
+// else `stride` elements per expert into the contiguous array (null if neither).
+// `e` is uniform over the workgroup, so this is scalar work.
+template <typename P>
+__device__ __forceinline__ const P* expert_operand(const void* base, const void* const* table,
+                                                   int e, int64_t stride) {
+  if (table) return (const P*)table[e];
+  return base ? (const P*)base + e * stride : nullptr;
+}
+
+// *p for a p that may come out of such a pointer table.  A pointer read from memory
+// has no known address space, and a plain load through it would be a flat load (it
+// waits on two counters and can reach LDS); this one says that p is global memory.
+template <int kBytes> struct BitsOf;
+template <> struct BitsOf<2> { typedef uint16_t type; };
+template <> struct BitsOf<4> { typedef uint32_t type; };
+template <> struct BitsOf<8> { typedef uint64_t type; };
+template <typename V>
+__device__ __forceinline__ V load_global(const void* p) {
+  typedef typename BitsOf<sizeof(V)>::type bits_t;
+  const bits_t b = *(__attribute__((address_space(1))) const bits_t*)p;
+  return __builtin_bit_cast(V, b);
+}
 
 // The part of the gelu'(-|x|) table the fused DGRAD epilogue keeps in LDS: the
 // bf16 patterns of 2^-28 <= |x| < 16, 4096 floats at a fixed place behind the

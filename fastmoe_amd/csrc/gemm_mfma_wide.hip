@@ -116,12 +116,12 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
   if (MODE == GEMM_FWD) {
     M = cnt; N = out_f; K = in_f;
     A = (const F*)g.a + row0 * in_f;                 lda = in_f;
-    B = (const F*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
+    B = expert_operand<F>(g.b, g.w_table, e, (int64_t)out_f * in_f); ldb = in_f;
     C = (F*)g.c + row0 * out_f;                      ldc = out_f;
   } else if (MODE == GEMM_DGRAD) {
     M = cnt; N = in_f; K = out_f;
     A = (const F*)g.a + row0 * out_f;                lda = out_f;
-    B = (const F*)g.b + (int64_t)e * out_f * in_f;   ldb = in_f;
+    B = expert_operand<F>(g.b, g.w_table, e, (int64_t)out_f * in_f); ldb = in_f;
     C = (F*)g.c + row0 * in_f;                       ldc = in_f;
   } else {
     M = out_f; N = in_f; K = cnt;
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
     __syncthreads();
   }
 
-  const F* bias = (MODE == GEMM_FWD && g.bias) ? (const F*)g.bias + (int64_t)e * out_f : nullptr;
+  const F* bias = MODE == GEMM_FWD ? expert_operand<F>(g.bias, g.bias_table, e, out_f) : nullptr;
   if constexpr (Mma::kSwap) {
     // 32x32 block, operands swapped: accumulator r of a lane is row lane % 32,
     // column 8 * (r / 4) + 4 * (lane / 32) + r % 4
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
           if (m < M && n < N) {  // N is a multiple of 4
             Vec4 o;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) o[c] = acc[i][j][4 * q + c] + (bias ? bias[n + c] : (F)0);
+            for (int c = 0; c < 4; ++c) o[c] = acc[i][j][4 * q + c] + (bias ? load_global<F>(bias + n + c) : (F)0);
             *reinterpret_cast<Vec4*>(C + (int64_t)m * ldc + n) = o;
           }
         }
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(kWideThreads, (WideMma<F>::kWaves)) void gemm_wide_
 #pragma unroll
     for (int j = 0; j < TB; ++j) {
       const int n = n0 + wave_n * 64 + j * BLK + lr;
-      const F bv = bias && n < N ? bias[n] : (F)0;
+      const F bv = bias && n < N ? load_global<F>(bias + n) : (F)0;
 #pragma unroll
       for (int i = 0; i < TB; ++i) {
 #pragma unroll

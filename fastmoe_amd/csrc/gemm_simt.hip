@@ -51,12 +51,12 @@ __global__ __launch_bounds__(STHREADS) void gemm_simt_kernel(GemmArgs g) {
   if (MODE == GEMM_FWD) {
     M = cnt; N = out_f; K = in_f;
     A = (const T*)g.a + row0 * in_f;                 sam = in_f;  sak = 1;
-    B = (const T*)g.b + (int64_t)e * out_f * in_f;   sbk = 1;     sbn = in_f;
+    B = expert_operand<T>(g.b, g.w_table, e, (int64_t)out_f * in_f); sbk = 1;     sbn = in_f;
     C = (T*)g.c + row0 * out_f;                      ldc = out_f;
   } else if (MODE == GEMM_DGRAD) {
     M = cnt; N = in_f; K = out_f;
     A = (const T*)g.a + row0 * out_f;                sam = out_f; sak = 1;
-    B = (const T*)g.b + (int64_t)e * out_f * in_f;   sbk = in_f;  sbn = 1;
+    B = expert_operand<T>(g.b, g.w_table, e, (int64_t)out_f * in_f); sbk = in_f;  sbn = 1;
     C = (T*)g.c + row0 * in_f;                       ldc = in_f;
   } else {
     M = out_f; N = in_f; K = cnt;
@@ -111,8 +111,7 @@ __global__ __launch_bounds__(STHREADS) void gemm_simt_kernel(GemmArgs g) {
     __syncthreads();
   }
 
-  const T* bias = (MODE == GEMM_FWD && g.bias)
-                      ? (const T*)g.bias + (int64_t)e * out_f : nullptr;
+  const T* bias = MODE == GEMM_FWD ? expert_operand<T>(g.bias, g.bias_table, e, out_f) : nullptr;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = m0 + ty * 4 + i;
@@ -122,7 +121,7 @@ __global__ __launch_bounds__(STHREADS) void gemm_simt_kernel(GemmArgs g) {
       const int n = n0 + tx * 4 + j;
       if (n >= N) continue;
       acc_t v = acc[i][j];
-      if (bias) v += Elem<T>::to_acc(bias[n]);
+      if (bias) v += Elem<T>::to_acc(load_global<T>(bias + n));
       C[(int64_t)m * ldc + n] = Elem<T>::from_acc(v);
     }
   }

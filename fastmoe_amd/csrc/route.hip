@@ -363,6 +363,13 @@ static int static_scratch(void** out) {
   return FMOE_OK;
 }
 
+// The routing share of fmoe_init(): looks up the current GPU's copy of the static
+// buffer, so that fmoe_route_static has no runtime query left to make.
+int route_static_init() {
+  void* p = nullptr;
+  return static_scratch(&p);
+}
+
 struct RouteWs {
   int32_t* block_hist;
   int32_t* cap_copy;

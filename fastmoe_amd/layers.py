@@ -155,21 +155,41 @@ class FMoE(nn.Module):
             self.gate_hook(gate_top_k_idx, gate_score, None)
 
         masked = self.mask is not None and self.mask_dict is not None
+        if self._device_side_dispatch():
+            # no host copy anywhere: counts stay in the RoutePlan
+            score = gate_score.reshape(-1, self.top_k)
+            if masked:
+                # masked tokens (fmoe/layers.py:240-251 deletes their rows, which
+                # needs their number on the host) keep their place and lose their
+                # slots instead: a slot of -1 is dropped by the routing kernels
+                mask = self.mask.view(-1).to(gate_top_k_idx.device)
+                gate_top_k_idx = torch.where((mask == 0).view(-1, 1),
+                                             gate_top_k_idx.view(-1, self.top_k), -1)
+            plan = RoutePlan(gate_top_k_idx, self.num_expert)
+            x = tree.map_structure(lambda t: FusedScatter.apply(t, plan), moe_inp)
+            x = tree.map_structure(lambda t: self._run_experts(t, plan.segments), x) \
+                if not self.experts_fused else self.experts(x, plan.segments)
+            out = tree.map_structure(
+                lambda t: FusedGatherCombine.apply(t, score, plan), x)
+            if masked:
+                # a masked token's k slots all hold mask_dict[mask value] (zero if the
+                # value has no entry), fmoe/layers.py:262-286: their score-weighted sum
+                # is (sum of the token's scores) x that row
+                total = score.sum(dim=-1, keepdim=True)
+
+                def fill(t):
+                    for k, v in self.mask_dict.items():
+                        row = (total * v.to(total.dtype).view(1, -1)).to(t.dtype)
+                        t = torch.where((mask == k).view(-1, 1), row, t)
+                    return t
+                out = tree.map_structure(fill, out)
+            return out
+
         if masked:
             mask = self.mask.view(-1)
             keep = mask == 0
             moe_inp = tree.map_structure(lambda t: t[keep, :], moe_inp)
             gate_top_k_idx = gate_top_k_idx[keep, :]
-
-        if not masked and self._device_side_dispatch():
-            # no host copy anywhere: counts stay in the RoutePlan
-            plan = RoutePlan(gate_top_k_idx, self.num_expert)
-            score = gate_score.reshape(-1, self.top_k)
-            x = tree.map_structure(lambda t: FusedScatter.apply(t, plan), moe_inp)
-            x = tree.map_structure(lambda t: self._run_experts(t, plan.segments), x) \
-                if not self.experts_fused else self.experts(x, plan.segments)
-            return tree.map_structure(
-                lambda t: FusedGatherCombine.apply(t, score, plan), x)
 
         fwd = _fmoe_general_global_forward(
             moe_inp, gate_top_k_idx, self.expert_fn, self.num_expert,

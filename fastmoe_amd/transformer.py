@@ -6,7 +6,17 @@ import torch.nn as nn
 
 from .functions import SegmentTable
 from .layers import FMoE
-from .linear import FMoELinear, MOELinear, act_linear, linear_act_linear
+from .linear import (FMoELinear, MOELinear, ParamTables, act_linear, linear_act_linear,
+                     linear_act_linear_list)
+
+
+def _watched(*modules) -> bool:
+    r"""Whether anybody has hooks on one of `modules` that only a call of the module
+    itself (forward hooks) or its own autograd nodes (backward hooks) would run."""
+    return any(m is not None and isinstance(m, nn.Module) and
+               (m._forward_hooks or m._forward_pre_hooks or m._backward_hooks or
+                getattr(m, "_backward_pre_hooks", None))
+               for m in modules)
 
 
 class _LinearView:
@@ -57,10 +67,11 @@ class _Expert(nn.Module):
         self.activation = activation
 
     def forward(self, inp, fwd_expert_count):
-        if any(m._forward_hooks or m._forward_pre_hooks for m in (self.htoh4, self.h4toh)):
-            # somebody watches the two linear modules: call them as modules
+        if _watched(self.htoh4, self.h4toh, self.activation):
+            # somebody watches the linear modules or the activation: call them as
+            # modules, the way the reference does (fmoe/transformer.py:25-33)
             x = self.htoh4(inp, fwd_expert_count)
-            if self.h4toh._forward_hooks or self.h4toh._forward_pre_hooks:
+            if _watched(self.h4toh, self.activation):
                 return self.h4toh(self.activation(x), fwd_expert_count)
             return act_linear(self.activation, x, fwd_expert_count, self.h4toh.weight,
                               self.h4toh.bias)
@@ -85,34 +96,51 @@ class _Expert(nn.Module):
     @staticmethod
     def can_run_list(experts) -> bool:
         r"""Whether `experts` (the reference's layout: one `_Expert(1, ...)` per
-        expert) can run as ONE grouped call on concatenated weights."""
+        expert) can run as ONE grouped call per layer on per-expert weight pointers:
+        single-expert modules of one shape, dtype and device, and nobody watching them
+        (hooks on a list module run only when that module is called, which the
+        reference-shaped route does)."""
         first = experts[0] if len(experts) else None
         if not isinstance(first, _Expert):
             return False
+        w1, w2 = first.htoh4.weight, first.h4toh.weight
         for e in experts:
             if not (isinstance(e, _Expert) and e.activation is first.activation
-                    and e.htoh4.in_feat == first.htoh4.in_feat
-                    and e.htoh4.out_feat == first.htoh4.out_feat
+                    and e.htoh4.num_expert == 1 and e.h4toh.num_expert == 1
+                    and e.htoh4.weight.shape == w1.shape and e.h4toh.weight.shape == w2.shape
                     and (e.htoh4.bias is None) == (first.htoh4.bias is None)
                     and (e.h4toh.bias is None) == (first.h4toh.bias is None)
-                    and e.htoh4.weight.dtype == first.htoh4.weight.dtype):
+                    and e.htoh4.weight.dtype == w1.dtype and e.h4toh.weight.dtype == w1.dtype
+                    and e.htoh4.weight.device == w1.device
+                    and e.h4toh.weight.device == w1.device
+                    and e.htoh4.weight.is_cuda
+                    and not _watched(e, e.htoh4, e.h4toh)):
                 return False
-        return True
+        return not _watched(first.activation)
 
     @staticmethod
     def run_list(experts, inp, segments: SegmentTable):
         r"""The modules of `experts` applied to their row segments in two grouped
-        GEMMs: the per-expert weights are concatenated to `[E, out, in]` for the
-        call (a copy of the weights per pass, autograd splits the gradients back),
-        and no count is read to the host."""
-        def cat(get):
-            parts = [get(e) for e in experts]
-            return None if parts[0] is None else torch.cat(parts, dim=0)
-
+        GEMMs that read every expert's weight where it lies (tables of per-expert
+        pointers, kept on the list and rebuilt only when a parameter's storage moves):
+        no weight is copied and no count is read to the host."""
+        tables = getattr(experts, "_fmoe_param_tables", None)
+        if tables is None:
+            tables = ParamTables()
+            try:
+                object.__setattr__(experts, "_fmoe_param_tables", tables)
+            except Exception:   # a plain list: no place to keep them
+                pass
         first = experts[0]
-        w1, b1 = cat(lambda e: e.htoh4.weight), cat(lambda e: e.htoh4.bias)
-        w2, b2 = cat(lambda e: e.h4toh.weight), cat(lambda e: e.h4toh.bias)
-        return linear_act_linear(first.activation, inp, segments, w1, b1, w2, b2)
+
+        def col(get):
+            parts = [get(e) for e in experts]
+            return None if parts[0] is None else parts
+
+        return linear_act_linear_list(
+            first.activation, inp, segments,
+            col(lambda e: e.htoh4.weight), col(lambda e: e.htoh4.bias),
+            col(lambda e: e.h4toh.weight), col(lambda e: e.h4toh.bias), tables)
 
 
 class FMoETransformerMLP(FMoE):
@@ -124,8 +152,9 @@ class FMoETransformerMLP(FMoE):
       weights are `[E, out, in]` tensors and runs the device-side dispatch;
       False builds `num_expert` single-expert modules as the reference does
       (state-dict keys `experts.<i>.htoh4.weight`); they still run as one
-      grouped call per layer without a host read, on weights concatenated per
-      pass.  Checkpoints in either layout load into either.
+      grouped call per layer without a host read, the kernels reading each
+      expert's weight through a pointer table (no copy).  Checkpoints in either
+      layout load into either.
     """
 
     def __init__(self, num_expert=32, d_model=1024, d_hidden=4096,

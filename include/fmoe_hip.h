@@ -58,6 +58,17 @@ typedef enum fmoe_dtype {
 const char* fmoe_version(void);
 const char* fmoe_last_error(void);
 
+/*
+ * Optional one-time set-up of the CURRENT GPU, on `stream` (waited for before the
+ * call returns): everything the entry points below otherwise do lazily at their
+ * first call on a GPU, namely the activation tables of the 16-bit kernels and the
+ * device address of fmoe_route_static's built-in buffer.  Callers that capture HIP
+ * graphs call it once per GPU before the first capture; everybody else may skip it.
+ * Thread-safe and idempotent.  No counterpart in the reference (its extension has
+ * no set-up of its own beyond the stream manager, cuda/stream_manager.cpp:75-93).
+ */
+int fmoe_init(void* stream);
+
 /* ------------------------------------------------------------------ routing */
 
 /*
@@ -111,8 +122,9 @@ int fmoe_route(const int64_t* gate, int64_t numel, int32_t n_expert,
  * the same results, with the per-block histograms in a buffer built into the library
  * (FMOE_ROUTE_STATIC_SCRATCH_BYTES per GPU, held until the process ends) instead
  * of a workspace argument.  It calls no allocating routine, so it may be used
- * under HIP graph capture, in serving loops and in harnesses that forbid
- * hipMalloc.  Sizes whose workspace (fmoe_route_workspace_bytes) exceeds the
+ * under HIP graph capture (after fmoe_init(), or one eager call, on that GPU: the
+ * first use on a GPU asks the runtime for the buffer's address), in serving loops
+ * and in harnesses that forbid hipMalloc.  Sizes whose workspace (fmoe_route_workspace_bytes) exceeds the
  * buffer are rejected with FMOE_ERR_WORKSPACE.  All calls on one GPU share the
  * buffer: calls that overlap in time on one GPU (two streams) race.
  * No counterpart in the reference; it exists for the callers named above.
@@ -258,9 +270,9 @@ int fmoe_grouped_linear_bwd(const void* dy, const void* x, const void* w,
  * leave the same output tiles (the activation kernel's own table of gelu(x) for
  * 16-bit x, applied to the rounded y: the same bits as fmoe_gelu_fwd over y); for
  * other dtypes and shapes, and below about 768 rows per expert (where the separate
- * kernel is as fast), the entry point runs that kernel behind the GEMM;
- * FMOE_FUSE_FWD_ACT=0 in the environment makes it do so always (a tuning aid).  Rows
- * of y_act behind seg_off[n_expert] are left untouched, like those of y.
+ * kernel is as fast), the entry point runs that kernel behind the GEMM
+ * (fmoe_set_gemm_path(6) makes it do so always).  Rows of y_act behind
+ * seg_off[n_expert] are left untouched, like those of y.
  */
 int fmoe_grouped_linear_fwd_act(const void* x, const void* w, const void* bias,
                                 const int32_t* seg_off, void* y, void* y_act,
@@ -284,6 +296,43 @@ int fmoe_grouped_linear_bwd_act(const void* dy, const void* x, const void* w,
                                 void* dx, void* dw, void* dbias, int64_t n_rows,
                                 int64_t in_feat, int64_t out_feat,
                                 int64_t n_expert, int dtype, void* stream);
+
+/*
+ * The grouped linear layer for experts whose parameters are SEPARATE allocations:
+ * the reference's FMoETransformerMLP keeps one single-expert module per expert
+ * (fmoe/transformer.py:51-55), and its GEMM loop addresses every expert's weight
+ * through a pointer of its own (cuda/parallel_linear.cuh:69-87).  w_ptrs and
+ * bias_ptrs (may be NULL) are DEVICE arrays of n_expert device pointers: expert e's
+ * weight [out_feat, in_feat] is at w_ptrs[e], its bias [out_feat] at bias_ptrs[e];
+ * every pointer 16-byte aligned.  Everything else is as in the entry points above:
+ *   _fwd_ptrs  = fmoe_grouped_linear_fwd, or with y_act != NULL
+ *                fmoe_grouped_linear_fwd_act;
+ *   _bwd_ptrs  = fmoe_grouped_linear_bwd, or with act_pre != NULL
+ *                fmoe_grouped_linear_bwd_act.  dw and dbias stay single [E, out, in]
+ *                and [E, out] arrays (the caller hands out per-expert views of them).
+ * No weight is copied, and the results carry the same bits as a call on the
+ * concatenated weights.
+ */
+int fmoe_grouped_linear_fwd_ptrs(const void* x, const void* const* w_ptrs,
+                                 const void* const* bias_ptrs, const int32_t* seg_off,
+                                 void* y, void* y_act, int64_t n_rows, int64_t in_feat,
+                                 int64_t out_feat, int64_t n_expert, int dtype,
+                                 void* stream);
+int fmoe_grouped_linear_bwd_ptrs(const void* dy, const void* x, const void* const* w_ptrs,
+                                 const int32_t* seg_off, const void* act_pre, void* dx,
+                                 void* dw, void* dbias, int64_t n_rows, int64_t in_feat,
+                                 int64_t out_feat, int64_t n_expert, int dtype,
+                                 void* stream);
+
+/*
+ * table[i] = host_ptrs[i] for i < n: fills a DEVICE array of pointers (the w_ptrs /
+ * bias_ptrs above) from a HOST array, asynchronously on `stream`; the values travel
+ * as kernel arguments, so the host array may be reused as soon as the call returns
+ * and nothing is synchronised.  The counterpart of the host-side pointer arithmetic
+ * of cuda/parallel_linear.cuh:69-87.
+ */
+int fmoe_pointer_table(const void* const* host_ptrs, int64_t n, const void** table,
+                       void* stream);
 
 /*
  * seg_off (device int32[E+1]) from HOST int64 counts, the form in which the
@@ -341,11 +390,14 @@ int fmoe_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n,
                   const int32_t* n_rows_dev, int64_t row_len, int dtype, void* stream);
 
 /*
- * Selects the grouped-GEMM kernel family: 0 = automatic (MFMA where the shape
- * allows, tile shape from the library's cost model), 1 = force the scalar
- * kernel, 2..5 = MFMA with bf16/f16 tile configuration 1..4 forced (256x256,
- * 128x256, 128x128, 256x256 with K slices of 64; f32/f64 have one tile shape).  A testing and tuning aid
- * with no counterpart in the reference; process-wide, not thread-safe.
+ * Selects the grouped-GEMM kernel family for the CALLING THREAD's later calls:
+ * 0 = automatic (MFMA where the shape allows, tile shape from the library's cost
+ * model), 1 = force the scalar kernel, 2..5 = MFMA with bf16/f16 tile
+ * configuration 1..4 forced (256x256, 128x256, 128x128, 256x256 with K slices of
+ * 64; f32/f64 have one tile shape), 6 = automatic, with the forward activation of
+ * fmoe_grouped_linear_fwd_act always as a kernel of its own.  A testing aid with
+ * no counterpart in the reference; the setting is thread-local (every thread
+ * starts at 0), so concurrent callers do not disturb each other.
  */
 int fmoe_set_gemm_path(int path);
 

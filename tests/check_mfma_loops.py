@@ -1,6 +1,6 @@
-"""Checks what the compiler made of the K loops of gemm_mfma.hip.
+"""Checks what the compiler made of the K loops of fastmoe_amd/csrc/gemm_mfma_impl.h.
 
-    python fastmoe_amd/csrc/check_mfma_loops.py [--all-dtypes] [--keep FILE.s]
+    python tests/check_mfma_loops.py [--all-dtypes] [--keep FILE.s]
 
 The kernels copy their operands into LDS with `buffer_load ... lds` written as inline
 assembly, and wait for them with their own `s_waitcnt vmcnt(n)`: the compiler does not
@@ -19,7 +19,7 @@ EPILOGUE, never to the loop itself):
 The script compiles the file to assembly for gfx950 (bf16 kernels only unless
 --all-dtypes: about 1.5 instead of 3.5 minutes), finds every loop with at least 16
 MFMAs and fewer than 700 lines, and reports the three counts; exit status 1 if any is
-not zero.
+not zero.  A `flat_load` anywhere in a kernel of the file is reported as well.
 """
 from __future__ import annotations
 
@@ -30,6 +30,8 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(os.path.dirname(HERE), "fastmoe_amd")
+CSRC = os.path.join(PKG, "csrc")
 
 
 def _library_build():
@@ -38,7 +40,7 @@ def _library_build():
     import importlib.util
 
     spec = importlib.util.spec_from_file_location(
-        "fmoe_library_build", os.path.join(os.path.dirname(HERE), "build.py"))
+        "fmoe_library_build", os.path.join(PKG, "build.py"))
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     return mod
@@ -47,19 +49,27 @@ def _library_build():
 def compile_to_assembly(out_path: str, all_dtypes: bool) -> None:
     _build = _library_build()
 
-    cmd = [_build.HIPCC, *_build.FLAGS, "--cuda-device-only", "-S",
-           os.path.join(HERE, "gemm_mfma.hip"), "-o", out_path]
-    if not all_dtypes:
-        cmd.insert(1, "-DFMOE_TUNING_BF16_ONLY")
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + res.stderr[-4000:])
+    # one translation unit per element type; their assembly is concatenated
+    units = ["gemm_mfma_bf16.hip"] + (["gemm_mfma_f16.hip"] if all_dtypes else [])
+    with open(out_path, "w") as out:
+        for unit in units:
+            part = out_path + "." + unit + ".s"
+            cmd = [_build.HIPCC, *_build.FLAGS, "--cuda-device-only", "-S",
+                   os.path.join(CSRC, unit), "-o", part]
+            res = subprocess.run(cmd, capture_output=True, text=True)
+            if res.returncode != 0:
+                raise RuntimeError("hipcc failed:\n" + res.stderr[-4000:])
+            with open(part) as f:
+                out.write(f.read())
+            os.remove(part)
 
 
 def scan(asm_text: str):
-    """[(kernel, [(mfmas, lines, compiler_vmcnt_waits, accvgpr_moves, scratch_ops)])]"""
+    """([(kernel, [(mfmas, lines, compiler_vmcnt_waits, accvgpr_moves, scratch_ops)])],
+    {kernel: flat loads anywhere in its body})"""
     lines = asm_text.split("\n")
     out = []
+    flat = {}
     for start in (i for i, l in enumerate(lines) if re.match(r"^_ZN4fmoe\S+:", l)):
         name = lines[start].split(":")[0]
         end = next((i for i in range(start, len(lines)) if lines[i].startswith(".Lfunc_end")),
@@ -67,6 +77,9 @@ def scan(asm_text: str):
         if end is None:
             continue
         body = lines[start:end]
+        n_flat = sum(1 for x in body if re.match(r"^\s+flat_load", x))
+        if n_flat:
+            flat[name] = n_flat
         labels = {}
         for i, l in enumerate(body):
             m = re.match(r"^(\.LBB\d+_\d+):", l)
@@ -95,7 +108,7 @@ def scan(asm_text: str):
             loops.append((mfmas, len(block), waits, moves, scratch))
         if loops:
             out.append((name, loops))
-    return out
+    return out, flat
 
 
 def main() -> int:
@@ -107,7 +120,7 @@ def main() -> int:
     if args.assembly:
         text = open(args.assembly).read()
     else:
-        build_dir = os.path.join(HERE, "build")      # the library's object directory
+        build_dir = os.path.join(CSRC, "build")      # the library's object directory
         os.makedirs(build_dir, exist_ok=True)
         path = args.keep or os.path.join(build_dir, "gemm_mfma_loops.%d.s" % os.getpid())
         try:
@@ -116,8 +129,15 @@ def main() -> int:
         finally:
             if not args.keep and os.path.exists(path):
                 os.remove(path)
-    found = scan(text)
+    found, flat = scan(text)
     bad = 0
+    # The activation epilogues index an LDS table with an offset that may lie outside
+    # the table (the result is then recomputed): harmless as an LDS read, a wild global
+    # read if the compiler ever lost the pointer's address space and emitted a flat load.
+    for name, n in flat.items():
+        print("%s: %d flat_load instructions (LDS / global pointers must keep their "
+              "address spaces)" % (name[:80], n))
+        bad += n
     for name, loops in found:
         short = re.sub(r"_ZN4fmoe\d+", "", name).replace("14__hip_bfloat16", "bf16")
         short = short.replace("6__half", "f16")[:64]

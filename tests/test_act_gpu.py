@@ -121,7 +121,7 @@ def test_live_row_hint_skips_dead_rows(dt):
     """With a device-side count of live rows only those rows are computed; the
     rest of the output is left as it was."""
     from fastmoe_amd import fmoe_cuda
-    from fastmoe_amd.fmoe_cuda import _L, _dt, _lib, _stream
+    from fastmoe_amd._ctypes_ops import _L, _dt, _lib, _stream
 
     dtype = DTYPES[dt]
     g = torch.Generator().manual_seed(5)

@@ -2,7 +2,8 @@
 reference's cuda/fmoe_cuda.cpp:104-125) against the ctypes module: the same C
 ABI underneath, so every operator must return bit-identical tensors; then the
 routing / dispatch / linear / layer suites once more in a child process with
-FMOE_BINDING=compiled, where the whole Python layer runs on the extension."""
+FMOE_BINDING=ctypes: the whole Python layer runs on the extension by default, and
+there on the ctypes calls."""
 import os
 import subprocess
 import sys
@@ -22,9 +23,11 @@ def _same(a, b):
 
 @pytest.mark.gpu
 def test_compiled_module_matches_the_ctypes_module_bit_for_bit():
-    from fastmoe_amd import _ext, fmoe_cuda as py
+    from fastmoe_amd import _ext, fmoe_cuda
 
+    py = fmoe_cuda.ctypes_ops
     cx = _ext.load()
+    assert fmoe_cuda.BINDING == "compiled"      # the default
     e, k, t, d, h = 6, 2, 300, 64, 96
     gate = torch.from_numpy(make_gate(t, k, e, drop=0.1, seed=3, empty=(4,))).cuda()
     # routing
@@ -101,12 +104,12 @@ def test_compiled_module_matches_the_ctypes_module_bit_for_bit():
 
 @pytest.mark.gpu
 @pytest.mark.timeout(900)
-def test_suites_pass_on_the_compiled_binding():
+def test_suites_pass_on_the_ctypes_binding():
     """Routing, dispatch, linear, activation and layer suites with the package bound
-    to the compiled extension (one child process; the big benchmark-size cases stay
-    with the default binding).  The activation suites also watch the per-op event
-    hook, which the compiled operators must feed like the ctypes ones."""
-    env = dict(os.environ, FMOE_BINDING="compiled")
+    to the ctypes calls instead of the compiled extension (one child process; the big
+    benchmark-size cases stay with the default binding).  The activation suites also
+    watch the per-op event hook, which both bindings must feed alike."""
+    env = dict(os.environ, FMOE_BINDING="ctypes")
     cmd = [sys.executable, "-m", "pytest", "-x", "-q", "-m", "gpu", "-p", "no:cacheprovider",
            "tests/test_routing_gpu.py", "tests/test_dispatch_gpu.py", "tests/test_linear_gpu.py",
            "tests/test_layer_gpu.py", "tests/test_act_gpu.py", "tests/test_fused_act_gpu.py",

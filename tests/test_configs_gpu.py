@@ -6,6 +6,7 @@ whole expert for the Mixtral-sized cfg4.  Tolerance: the bf16 bound 2e-2, both
 norm-wise and row by row.  Also the reference-shaped dispatch (MOEScatter /
 MOEGather, module-list experts) through autograd, and nested (dict / list)
 inputs as in tests/test_mimo.py."""
+import numpy as np
 import pytest
 import torch
 import torch.nn.functional as F
@@ -408,3 +409,150 @@ def test_nested_inputs_as_in_the_reference_mimo_suite(num_expert, top_k, dt, lis
     # the second entry never reaches the gate: its gradient is the experts' share
     # alone, 2/3 of what the oracle's 3 x sum() sends back to x
     assert b.grad is not None and max_rel_err(b.grad, x_cpu.grad * (2.0 / 3.0)) <= tol
+
+
+def _masked_reference(moe, x, mask, mask_dict):
+    """Dense float64 restatement of the masked layer (fmoe/layers.py:240-295): masked
+    tokens take no expert; each of their k slots holds mask_dict[mask value] (zeros
+    without an entry); the combine weights every slot by the gate's score."""
+    from oracle import moe_oracle as O
+
+    with torch.no_grad():
+        idx, score = moe.gate(x.cuda())
+    idx, score = idx.cpu(), score.double().cpu().reshape(x.shape[0], -1)
+    ex = moe.experts
+    params = [p.detach().double().cpu().requires_grad_(True)
+              for p in (ex.htoh4.weight, ex.htoh4.bias, ex.h4toh.weight, ex.h4toh.bias)]
+    xd = x.double().cpu().requires_grad_(True)
+    sd = score.clone().requires_grad_(True)
+    live_idx = torch.where((mask == 0).view(-1, 1), idx, torch.full_like(idx, -1))
+    out = O.brute_force_moe_mlp(xd, live_idx, sd, *params)
+    for k, v in mask_dict.items():
+        row = sd.sum(dim=1, keepdim=True) * v.double().cpu().view(1, -1)
+        out = torch.where((mask == k).view(-1, 1), row, out)
+    return out, xd, sd, params
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_masked_layer_dispatches_on_the_device(fused):
+    """mask / mask_dict (fmoe/layers.py:240-255,270-286) without the reference's
+    row deletion: masked tokens lose their slots inside the routing kernels, their
+    output rows come from mask_dict, and no call of the pass synchronises with the
+    host.  Outputs and gradients against the dense restatement."""
+    from fastmoe_amd import FMoETransformerMLP
+
+    torch.manual_seed(11)
+    t, d, h, e, k = 257, 64, 96, 5, 2
+    mask = torch.zeros(t, dtype=torch.long)
+    mask[3::7] = 1          # rows replaced by mask_dict[1]
+    mask[5::11] = 2         # rows replaced by mask_dict[2]
+    mask[6::13] = 3         # no entry: rows of zeros
+    mask_dict = {1: torch.randn(d).cuda(), 2: torch.zeros(d).cuda()}
+    moe = FMoETransformerMLP(e, d, h, top_k=k, mask=mask.cuda(), mask_dict=mask_dict,
+                             fused=True).cuda()
+    if not fused:
+        plain = FMoETransformerMLP(e, d, h, top_k=k, mask=mask.cuda(), mask_dict=mask_dict,
+                                   fused=False).cuda()
+        plain.load_state_dict(moe.state_dict())
+    else:
+        plain = moe
+    assert plain._device_side_dispatch()
+    x = torch.randn(t, d)
+    dy = torch.randn(t, d)
+    a = x.clone().cuda().requires_grad_(True)
+    dy_dev = dy.cuda()
+    plain(a).backward(dy_dev)                    # warm-up (tables, attributes)
+    a.grad = None
+    for p in plain.parameters():
+        p.grad = None
+    # the gate's own path to x is kept out of the comparison: the scores become a leaf
+    leaf = {}
+
+    def cut(m, i, o):
+        leaf["score"] = o[1].detach().requires_grad_(True)
+        return o[0], leaf["score"]
+    hook = plain.gate.register_forward_hook(cut)
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("error")      # any host synchronisation raises
+    try:
+        out = plain(a)
+        out.backward(dy_dev)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+        hook.remove()
+    want, xd, sd, params = _masked_reference(moe, x, mask, mask_dict)
+    want.backward(dy.double())
+    assert max_rel_err(out, want) <= 2e-5
+    assert not out[mask == 3].any().item() and not out[mask == 2].any().item()
+    assert max_rel_err(a.grad, xd.grad) <= 2e-5
+    assert not a.grad[mask != 0].any().item()    # masked tokens reach no expert
+    if fused:
+        got = [moe.experts.htoh4.weight.grad, moe.experts.htoh4.bias.grad,
+               moe.experts.h4toh.weight.grad, moe.experts.h4toh.bias.grad]
+    else:
+        got = [torch.cat([getattr(getattr(m, lin), par).grad for m in plain.experts])
+               for lin, par in (("htoh4", "weight"), ("htoh4", "bias"), ("h4toh", "weight"),
+                                ("h4toh", "bias"))]
+    for g, p in zip(got, params):
+        assert max_rel_err(g, p.grad) <= 2e-5
+    # the score gradient of a masked token is <dy, its mask_dict row>
+    assert max_rel_err(leaf["score"].grad.reshape(t, k), sd.grad) <= 2e-5
+    assert leaf["score"].grad.reshape(t, k)[mask == 1].any().item()
+
+
+def test_list_of_experts_with_hooks_takes_the_reference_route():
+    """A forward hook on one module of the list must run: the grouped call on pointer
+    tables never calls the modules, so such a list is dispatched the reference's way."""
+    from fastmoe_amd import FMoETransformerMLP
+
+    torch.manual_seed(5)
+    plain = FMoETransformerMLP(4, 32, 64, top_k=2, fused=False).cuda()
+    assert plain._device_side_dispatch()
+    calls = []
+    h = plain.experts[2].htoh4.register_forward_hook(lambda m, i, o: calls.append(2))
+    try:
+        assert not plain._device_side_dispatch()
+        x = torch.randn(50, 32, device="cuda")
+        want = plain(x)
+    finally:
+        h.remove()
+    assert calls and plain._device_side_dispatch()
+    assert max_rel_err(plain(x), want) <= 2e-5
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32", "f64"])
+def test_pointer_table_ops_give_the_bits_of_the_stacked_call(dt):
+    """fmoe_grouped_linear_{fwd,bwd}_ptrs on separately allocated per-expert weights
+    against the same call on their concatenation (cuda/parallel_linear.cuh:69-87 takes
+    per-expert pointers the same way): identical bits, every product, with and without
+    the activation."""
+    from fastmoe_amd import fmoe_cuda
+    from helpers import DTYPES, randn
+
+    dtype = DTYPES[dt]
+    counts = [300, 0, 129, 64, 1, 0, 513]
+    e, in_f, out_f = len(counts), 72, 136
+    seg = torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32).cuda()
+    n = sum(counts)
+    x = randn((n, in_f), dtype, 1).cuda()
+    dy = randn((n, out_f), dtype, 2).cuda()
+    ws = [randn((1, out_f, in_f), dtype, 10 + i, 0.1).cuda() for i in range(e)]
+    bs = [randn((1, out_f), dtype, 30 + i).cuda() for i in range(e)]
+    w, b = torch.cat(ws), torch.cat(bs)
+    wt, bt = fmoe_cuda.pointer_table(ws), fmoe_cuda.pointer_table(bs)
+    assert wt.dtype == torch.int64 and wt.tolist() == [t.data_ptr() for t in ws]
+    y = fmoe_cuda.grouped_linear_fwd(x, seg, w, b)
+    assert torch.equal(fmoe_cuda.grouped_linear_fwd_ptrs(x, seg, wt, bt, out_f), y)
+    assert torch.equal(fmoe_cuda.grouped_linear_fwd_ptrs(x, seg, wt, None, out_f),
+                       fmoe_cuda.grouped_linear_fwd(x, seg, w, None))
+    ya, aa = fmoe_cuda.grouped_linear_fwd(x, seg, w, b, with_gelu=True)
+    yb, ab = fmoe_cuda.grouped_linear_fwd_ptrs(x, seg, wt, bt, out_f, with_gelu=True)
+    assert torch.equal(ya, yb) and torch.equal(aa, ab)
+    for act_pre in (None, randn((n, in_f), dtype, 3).cuda()):
+        ga = fmoe_cuda.grouped_linear_bwd(dy, x, seg, w, act_pre=act_pre)
+        gb = fmoe_cuda.grouped_linear_bwd_ptrs(dy, x, seg, wt, act_pre=act_pre)
+        for p, q in zip(ga, gb):
+            assert p.shape == q.shape and torch.equal(p, q)
+    only_dx = fmoe_cuda.grouped_linear_bwd_ptrs(dy, x, seg, wt, need_bias=False, need_dw=False)
+    assert only_dx[1] is None and only_dx[2] is None
+    assert torch.equal(only_dx[0], fmoe_cuda.grouped_linear_bwd(dy, x, seg, w)[0])

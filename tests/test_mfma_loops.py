@@ -1,6 +1,6 @@
 """The K loops of the matrix-core GEMM as the compiler emits them: no wait of the
 compiler's own on the memory counter, no accumulator moves, no scratch access (see
-fastmoe_amd/csrc/check_mfma_loops.py for why each of them is expensive here).  Needs
+tests/check_mfma_loops.py for why each of them is expensive here).  Needs
 hipcc but no GPU; about a minute and a half."""
 import os
 import subprocess
@@ -16,8 +16,7 @@ def test_compiler_leaves_the_mfma_loops_alone():
 
     if not os.path.exists(lib_build.HIPCC):
         pytest.skip("no hipcc on this machine")
-    res = subprocess.run([sys.executable, os.path.join(ROOT, "fastmoe_amd", "csrc",
-                                                       "check_mfma_loops.py")],
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "check_mfma_loops.py")],
                          capture_output=True, text=True, timeout=900)
     assert res.returncode == 0, (res.stdout + res.stderr)[-3000:]
     assert " 0 flagged" in res.stdout
