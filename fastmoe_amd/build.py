@@ -40,6 +40,13 @@ FLAGS = [
 ]
 
 
+# Extra compiler flags for experiments with the kernels' named constants, e.g.
+# FMOE_EXTRA_HIPCC_FLAGS="-DFMOE_PATCH_ROWS=8 -DFMOE_PATCH_COLS=4" (the order in which
+# a launch walks its tiles); they enter the digest, so a library built with them is
+# never mistaken for the plain one.
+EXTRA_FLAGS = os.environ.get("FMOE_EXTRA_HIPCC_FLAGS", "").split()
+
+
 def source_hash() -> str:
     """Digest (12 hex digits) of every source and header the library is built from."""
     import hashlib
@@ -48,6 +55,8 @@ def source_hash() -> str:
     for name in SOURCES + HEADERS:
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(name.encode() + b"\0" + f.read() + b"\0")
+    if EXTRA_FLAGS:
+        h.update(" ".join(EXTRA_FLAGS).encode())
     return h.hexdigest()[:12]
 
 
@@ -64,7 +73,7 @@ def built_hash(lib_path: str = LIB_PATH):
 
 def _compile(src: str, verbose: bool) -> str:
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     if src == "api.hip":
         cmd.insert(-4, f'-DFMOE_SOURCE_HASH="{source_hash()}"')
     if verbose:

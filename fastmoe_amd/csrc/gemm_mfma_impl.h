@@ -123,10 +123,14 @@ template <> struct PackPair<__half> {
 // Fast form: `tab` is the slice of the table in LDS, valid for patterns whose
 // index (pattern without sign - kActTabFirst) is below kActTabCount.  The OR of
 // all indices goes into `seen`: a bit at or above kActTabCount's says that some
-// argument was outside and the result must be recomputed by the slow form (an
-// LDS read outside the slice returns whatever is there, or zero, never faults).
+// argument was outside and the result must be recomputed by the slow form.  `tab`
+// is typed as an LDS pointer, so the read with such an index is an LDS instruction
+// whatever the compiler makes of the code around it: outside the slice it returns
+// whatever is there, or zero, and never faults (a flat load could).
+typedef __attribute__((address_space(3))) const float* lds_float_ptr_t;
+typedef __attribute__((address_space(3))) const uint16_t* lds_u16_ptr_t;
 template <typename T>
-__device__ __forceinline__ uint32_t gelu_bwd_pair_fast(uint32_t h, uint32_t p, const float* tab,
+__device__ __forceinline__ uint32_t gelu_bwd_pair_fast(uint32_t h, uint32_t p, lds_float_ptr_t tab,
                                                        uint32_t& seen) {
   const uint32_t i0 = (p & 0x7fffu) - kActTabFirst, i1 = ((p >> 16) & 0x7fffu) - kActTabFirst;
   seen |= i0 | i1;
@@ -339,18 +343,24 @@ constexpr int kXcdRun = 32;
 // column.  32 consecutive numbers are a 4x8 patch (12 operand tiles for 32
 // products), 256 consecutive ones a 16x16 region.  Ragged edges shrink the
 // band, block or patch; the order stays a bijection.
+#ifndef FMOE_PATCH_ROWS
+#define FMOE_PATCH_ROWS 4
+#define FMOE_PATCH_COLS 8
+#define FMOE_BAND_ROWS 16
+#endif
 __device__ __forceinline__ void tile_order(int t, int rows, int cols, int& row, int& col) {
-  const int band = t / (16 * cols);
-  int r = t % (16 * cols);
-  const int band_rows = min(16, rows - band * 16);
-  const int blk = r / (band_rows * 8);
-  r %= band_rows * 8;
-  const int blk_cols = min(8, cols - blk * 8);
-  const int patch = r / (4 * blk_cols);
-  r %= 4 * blk_cols;
-  const int patch_rows = min(4, band_rows - patch * 4);
-  row = band * 16 + patch * 4 + r % patch_rows;
-  col = blk * 8 + r / patch_rows;
+  constexpr int kBand = FMOE_BAND_ROWS, kCols = FMOE_PATCH_COLS, kRows = FMOE_PATCH_ROWS;
+  const int band = t / (kBand * cols);
+  int r = t % (kBand * cols);
+  const int band_rows = min(kBand, rows - band * kBand);
+  const int blk = r / (band_rows * kCols);
+  r %= band_rows * kCols;
+  const int blk_cols = min(kCols, cols - blk * kCols);
+  const int patch = r / (kRows * blk_cols);
+  r %= kRows * blk_cols;
+  const int patch_rows = min(kRows, band_rows - patch * kRows);
+  row = band * kBand + patch * kRows + r % patch_rows;
+  col = blk * kCols + r / patch_rows;
 }
 
 // Where a tile sits in the rows of its expert.
@@ -742,8 +752,12 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
   // that range (zeros, denormals, |x| >= 16, infinities, NaNs) is looked up in the
   // full table in memory.
   constexpr bool fuse_fwd = MODE == GEMM_FWD_ACT;
-  uint16_t* fwd_tab = smem + kActTabLdsOffset / 2;
-  static_assert(BM * kLdc * 2 <= kActTabLdsOffset, "the table sits behind the largest staged tile");
+  // (behind this instantiation's own staged tile: a small tile shape then needs little
+  // LDS and two of its workgroups fit a CU)
+  constexpr int kTabOffset = BM * kLdc * 2;
+  static_assert(kTabOffset % 16 == 0 && kTabOffset <= kActTabLdsOffset, "place of the table");
+  uint16_t* fwd_tab_w = smem + kTabOffset / 2;
+  const lds_u16_ptr_t fwd_tab = (lds_u16_ptr_t)fwd_tab_w;
   static_assert((kActTabBytes / 16) % NT == 0, "the table splits evenly over the threads");
   constexpr int kTabPerThread = kActTabBytes / 16 / NT;
   i32x4_t tab_regs[kTabPerThread];
@@ -807,7 +821,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
     if constexpr (fuse_fwd) {
 #pragma unroll
       for (int i = 0; i < kTabPerThread; ++i)
-        reinterpret_cast<i32x4_t*>(fwd_tab)[tid + i * NT] = tab_regs[i];
+        reinterpret_cast<i32x4_t*>(fwd_tab_w)[tid + i * NT] = tab_regs[i];
     }
     __syncthreads();
     // Every pack gets registers of its own: a store holds its data registers
@@ -856,7 +870,7 @@ __device__ __forceinline__ void gemm_tile16(const GemmArgs& g, uint16_t* smem, T
     if constexpr (fuse_fwd) {
 #pragma unroll
       for (int i = 0; i < kTabPerThread; ++i)
-        reinterpret_cast<i32x4_t*>(fwd_tab)[tid + i * NT] = tab_regs[i];
+        reinterpret_cast<i32x4_t*>(fwd_tab_w)[tid + i * NT] = tab_regs[i];
     }
     __syncthreads();
     i32x4_t v[kSteps], w[kSteps];
@@ -1196,8 +1210,10 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   // DGRAD with the activation's backward fused in: the slice of the gelu' table
   // goes into LDS behind the staged tile (its loads fly during the staging)
   constexpr bool fuse_act = MODE == GEMM_DGRAD_ACT;
-  static_assert(BM * kLdc * 2 <= kActTabLdsOffset, "the table sits behind the largest staged tile");
-  float* act_tab = reinterpret_cast<float*>(smem + kActTabLdsOffset / 2);
+  constexpr int kTabOffset = BM * kLdc * 2;   // behind this instantiation's own staged tile
+  static_assert(kTabOffset % 16 == 0 && kTabOffset <= kActTabLdsOffset, "place of the table");
+  float* act_tab_w = reinterpret_cast<float*>(smem + kTabOffset / 2);
+  const lds_float_ptr_t act_tab = (lds_float_ptr_t)act_tab_w;
   // (an even split: a guarded load into the array would put it into scratch
   // memory, one load and one wait at a time)
   static_assert((kActTabCount / 4) % NT == 0, "the table splits evenly over the threads");
@@ -1272,7 +1288,7 @@ __device__ __forceinline__ void gemm_tile32(const GemmArgs& g, uint16_t* smem, T
   if constexpr (fuse_act) {
 #pragma unroll
     for (int i = 0; i < kTabPerThread; ++i)
-      reinterpret_cast<i32x4_t*>(act_tab)[tid + i * NT] = tab_regs[i];
+      reinterpret_cast<i32x4_t*>(act_tab_w)[tid + i * NT] = tab_regs[i];
   }
   if constexpr (kOverlap) {
     if constexpr (!fuse_act) {
@@ -1464,11 +1480,35 @@ __device__ __forceinline__ void edge_aware_tile(const GemmArgs& g, uint16_t* sme
 // many CUs then share the streaming.  It pays from K = 2048 on (measured on the
 // cfg-2 shapes from cold caches: K = 4096 forward 209 -> 180 us, dX 199 -> 182 us;
 // at K = 1024 the fixed cost of four times as many tiles eats the gain).
+// Their K slices hold 64 values: a narrow tile has 4 to 16 MFMAs per wave and K step,
+// and with slices of 32 its K loop ran at the pace of the per-slice barrier and wait
+// rather than of its copies (measured on the cfg-2 shapes with +-3 % ragged experts:
+// forward K = 4096 136 -> 128 us, dX K = 4096 151 -> 143 us, fused backward 325 ->
+// 311 us; nothing changes where no narrow tiles run).
 constexpr int kNarrowMax = 128;
 constexpr int kNarrowMinK = 2048;
+constexpr int kNarrowBK = 64;
+constexpr int kNarrowStages = 5;   // of a 64-row narrow tile (three slices of 64 in flight)
 template <int BM, int BN, int MODE>
 constexpr int narrow_factor() {
   return (BM == 256 && BN == 256 && MODE != GEMM_WGRAD) ? (is_fwd(MODE) ? 4 : 2) : 1;
+}
+
+// LDS bytes the remainder tiles of a BM x BN kernel need for their pipelines (their
+// staged output tiles are smaller than the main tile's): the 64- and 128-row tiles
+// of full width and, where the product has them, the narrow ones.
+template <int BM, int BN, int MODE>
+constexpr size_t remainder_lds_bytes() {
+  if (!has_small_tiles<BM, BN, MODE>()) return 0;
+  size_t need = (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2;
+  if (BM >= 4 * kSmallRows)
+    need = std::max(need, (size_t)4 * (2 * kSmallRows + BN) * kSmallBK * 2);
+  constexpr int kF = narrow_factor<BM, BN, MODE>();
+  if (kF > 1) {
+    need = std::max(need, (size_t)4 * (2 * kSmallRows + BN / kF) * kNarrowBK * 2);
+    need = std::max(need, (size_t)kNarrowStages * (kSmallRows + BN / kF) * kNarrowBK * 2);
+  }
+  return need;
 }
 
 // Runs the remainder tile at rows [where.m0, where.cnt) of its expert; n_tile
@@ -1481,9 +1521,10 @@ __device__ __forceinline__ void remainder_tile(const GemmArgs& g, uint16_t* smem
     if (narrow) {
       constexpr int NB = BN / kF;
       if (where.cnt - where.m0 > kSmallRows)
-        gemm_tile<T, 2 * kSmallRows, NB, kSmallBK, 2, 2, 4, MODE>(g, smem, where, n_tile * NB);
+        gemm_tile<T, 2 * kSmallRows, NB, kNarrowBK, 2, 2, 4, MODE>(g, smem, where, n_tile * NB);
       else
-        gemm_tile<T, kSmallRows, NB, kSmallBK, 2, 2, 8, MODE>(g, smem, where, n_tile * NB);
+        gemm_tile<T, kSmallRows, NB, kNarrowBK, 2, 2, kNarrowStages, MODE>(g, smem, where,
+                                                                         n_tile * NB);
       return;
     }
   }
@@ -1756,20 +1797,14 @@ static int launch_cfg(const GemmArgs& g, hipStream_t s) {
   using ATile = DmaTile<BM, BK, NW, MODE != GEMM_WGRAD>;
   using BTile = DmaTile<BN, BK, NW, is_fwd(MODE)>;
   constexpr size_t pipe_bytes = NS * (ATile::kBytes + BTile::kBytes);
-  // staged output tile (+ the activation table of a fused DGRAD epilogue)
-  constexpr size_t out_bytes =
-      MODE == GEMM_DGRAD_ACT ? (size_t)kActTabLdsOffset + kActTabBytes : (size_t)BM * (BN + 8) * 2;
-  constexpr size_t small_bytes = has_small_tiles<BM, BN, MODE>()
-      ? (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2 : 0;
+  // staged output tile (+ the activation table slice of a fused epilogue behind it)
+  constexpr size_t out_bytes = (size_t)BM * (BN + 8) * 2 +
+      (MODE == GEMM_DGRAD_ACT || MODE == GEMM_FWD_ACT ? (size_t)kActTabBytes : 0);
+  constexpr size_t small_bytes = remainder_lds_bytes<BM, BN, MODE>();
   constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
   constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
-  // a forward launch with the activation fused in keeps the table slice behind the
-  // place of the largest staged tile, whatever its own tile shape
-  constexpr size_t act_bytes = (size_t)kActTabLdsOffset + kActTabBytes;
-  constexpr size_t lds_max =
-      MODE == GEMM_FWD_ACT && act_bytes > lds_bytes ? act_bytes : lds_bytes;
-  static_assert(lds_max + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");
+  constexpr size_t lds_max = lds_bytes;
   constexpr size_t lds_launch = lds_max;
   auto kern = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, NS, MODE>;
   FMOE_SET_DYNAMIC_LDS_ONCE(kern, lds_max);
@@ -1868,7 +1903,7 @@ static int launch_bwd_fused(const GemmArgs& gd, const GemmArgs& gw, hipStream_t 
   constexpr int BM = 256, BN = 256, WM = 2, WN = 2, NT = WM * WN * 64;
   constexpr size_t pipe_bytes = (size_t)NS * (BM + BN) * BK * 2;
   constexpr size_t out_bytes = (size_t)kActTabLdsOffset + kActTabBytes;
-  constexpr size_t small_bytes = (size_t)kSmallStages * (kSmallRows + BN) * kSmallBK * 2;
+  constexpr size_t small_bytes = remainder_lds_bytes<BM, BN, GEMM_DGRAD>();
   constexpr size_t big_bytes = pipe_bytes > out_bytes ? pipe_bytes : out_bytes;
   constexpr size_t lds_bytes = big_bytes > small_bytes ? big_bytes : small_bytes;
   static_assert(lds_bytes + 1024 <= 160 * 1024, "LDS budget of a gfx950 CU");

@@ -165,12 +165,17 @@ class FMoE(nn.Module):
                 mask = self.mask.view(-1).to(gate_top_k_idx.device)
                 gate_top_k_idx = torch.where((mask == 0).view(-1, 1),
                                              gate_top_k_idx.view(-1, self.top_k), -1)
-            plan = RoutePlan(gate_top_k_idx, self.num_expert)
-            x = tree.map_structure(lambda t: FusedScatter.apply(t, plan), moe_inp)
-            x = tree.map_structure(lambda t: self._run_experts(t, plan.segments), x) \
-                if not self.experts_fused else self.experts(x, plan.segments)
-            out = tree.map_structure(
-                lambda t: FusedGatherCombine.apply(t, score, plan), x)
+            whole = getattr(self.experts, "can_run_layer", None) if self.experts_fused else None
+            if whole is not None and whole(moe_inp, self.top_k):
+                # dispatch, experts and combine as one autograd node (least host time)
+                out = self.experts.run_layer(moe_inp, gate_top_k_idx, score)
+            else:
+                plan = RoutePlan(gate_top_k_idx, self.num_expert)
+                x = tree.map_structure(lambda t: FusedScatter.apply(t, plan), moe_inp)
+                x = tree.map_structure(lambda t: self._run_experts(t, plan.segments), x) \
+                    if not self.experts_fused else self.experts(x, plan.segments)
+                out = tree.map_structure(
+                    lambda t: FusedGatherCombine.apply(t, score, plan), x)
             if masked:
                 # a masked token's k slots all hold mask_dict[mask value] (zero if the
                 # value has no entry), fmoe/layers.py:262-286: their score-weighted sum

@@ -3,11 +3,13 @@ from __future__ import annotations
 
 import torch
 import torch.nn as nn
+from torch.autograd import Function
 
+from . import fmoe_cuda
 from .functions import SegmentTable
 from .layers import FMoE
-from .linear import (FMoELinear, MOELinear, ParamTables, act_linear, linear_act_linear,
-                     linear_act_linear_list)
+from .linear import (FMoELinear, MOELinear, ParamTables, act_linear, is_exact_gelu,
+                     linear_act_linear, linear_act_linear_list)
 
 
 def _watched(*modules) -> bool:
@@ -17,6 +19,52 @@ def _watched(*modules) -> bool:
                (m._forward_hooks or m._forward_pre_hooks or m._backward_hooks or
                 getattr(m, "_backward_pre_hooks", None))
                for m in modules)
+
+
+class FusedExpertLayer(Function):
+    r"""The whole dispatch of a layer of GELU expert MLPs as ONE autograd node:
+    route -> scatter -> linear + GELU -> linear -> gather fused with the top-k
+    combine (fmoe/layers.py:26-78,281-295 around fmoe/transformer.py:25-33), and the
+    mirror image backwards.  The same kernels, in the same order, as the chain of
+    FusedScatter / MOELinearGelu / MOEGeluLinear / FusedGatherCombine nodes; what
+    it saves is host time (one node instead of four, no intermediate Python
+    objects), which is all a small layer costs."""
+
+    @staticmethod
+    def forward(ctx, inp, gate_idx, score, w1, b1, w2, b2):
+        top_k = gate_idx.shape[-1] if gate_idx.dim() >= 2 else 1
+        n_tokens = inp.shape[0]
+        with torch.no_grad():
+            pos, _counts, seg_off, inv = fmoe_cuda.route(gate_idx.contiguous(), w1.shape[0])
+        x = inp.contiguous()
+        if 4 <= top_k <= 64:
+            buf = fmoe_cuda.scatter_tokens(x, inv, top_k)
+        else:
+            buf = fmoe_cuda.local_scatter(x, pos, top_k, seg_off[-1:])
+        pre, act = fmoe_cuda.grouped_linear_fwd(buf, seg_off, w1, b1, with_gelu=True)
+        out_buf = fmoe_cuda.grouped_linear_fwd(act, seg_off, w2, b2)
+        ctx.score_like = (score.shape, score.dtype)
+        score = score.reshape(n_tokens, top_k).contiguous().to(out_buf.dtype)
+        ctx.top_k, ctx.n_tokens = top_k, n_tokens
+        ctx.has_bias = (b1 is not None, b2 is not None)
+        ctx.save_for_backward(buf, pre, act, out_buf, score, seg_off, inv, w1, w2)
+        return fmoe_cuda.gather_combine_fwd(out_buf, inv, score, n_tokens, top_k)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        buf, pre, act, out_buf, score, seg_off, inv, w1, w2 = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        d_out, dscore = fmoe_cuda.gather_combine_bwd(grad_y.contiguous(), out_buf, inv, score,
+                                                     ctx.n_tokens, ctx.top_k)
+        dpre, dw2, db2 = fmoe_cuda.grouped_linear_bwd(
+            d_out, act, seg_off, w2, need_bias=need[6] and ctx.has_bias[1], need_dx=True,
+            need_dw=need[5], act_pre=pre)
+        dbuf, dw1, db1 = fmoe_cuda.grouped_linear_bwd(
+            dpre, buf, seg_off, w1, need_bias=need[4] and ctx.has_bias[0], need_dx=need[0],
+            need_dw=need[3])
+        dx = fmoe_cuda.scatter_reduce(dbuf, inv, ctx.n_tokens, ctx.top_k) if need[0] else None
+        dscore = dscore.reshape(ctx.score_like[0]).to(ctx.score_like[1]) if need[2] else None
+        return dx, None, dscore, dw1, db1, dw2, db2
 
 
 class _LinearView:
@@ -79,6 +127,22 @@ class _Expert(nn.Module):
         # backward runs inside the second layer's backward kernel
         return linear_act_linear(self.activation, inp, fwd_expert_count, self.htoh4.weight,
                                  self.htoh4.bias, self.h4toh.weight, self.h4toh.bias)
+
+    def can_run_layer(self, inp, top_k) -> bool:
+        r"""Whether the whole layer (dispatch included) can run as one autograd node:
+        one 2-d GPU tensor in the parameters' dtype, the exact GELU between the two
+        layers, and nobody watching the modules inside."""
+        w1, w2 = self.htoh4.weight, self.h4toh.weight
+        return (torch.is_tensor(inp) and inp.dim() == 2 and inp.is_cuda
+                and inp.dtype == w1.dtype == w2.dtype and 1 <= top_k <= 64
+                and is_exact_gelu(self.activation, inp)
+                and not _watched(self, self.htoh4, self.h4toh, self.activation))
+
+    def run_layer(self, inp, gate_idx, score):
+        r"""`sum_j score[t, j] * expert_{gate_idx[t, j]}(inp[t])` over the live slots,
+        as one autograd node (FusedExpertLayer)."""
+        return FusedExpertLayer.apply(inp, gate_idx, score, self.htoh4.weight, self.htoh4.bias,
+                                      self.h4toh.weight, self.h4toh.bias)
 
     def __len__(self):
         return self.htoh4.num_expert

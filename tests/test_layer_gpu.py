@@ -358,3 +358,41 @@ def test_config2_full_size_layer_against_brute_force():
         hook.remove()
     assert max_rel_err(x2.grad, x_cpu.grad) <= tol
     assert max_row_rel_err(x2.grad, x_cpu.grad) <= 3e-2
+
+
+@pytest.mark.parametrize("dt,top_k", [("bf16", 2), ("f32", 3), ("bf16", 8)])
+def test_whole_layer_node_matches_the_chain_of_nodes(dt, top_k):
+    """FusedExpertLayer (dispatch, experts and combine as one autograd node) runs the
+    same kernels in the same order as the chain FusedScatter -> MOELinearGelu ->
+    MOEGeluLinear -> FusedGatherCombine: identical bits in the output and in every
+    gradient.  A hook on the activation module switches the single node off."""
+    from fastmoe_amd import FMoETransformerMLP
+
+    dtype = DTYPES[dt]
+    torch.manual_seed(9)
+    moe = FMoETransformerMLP(12, 64, 96, top_k=top_k).to(dtype).cuda()
+    x = torch.randn(200, 64, device="cuda").to(dtype)
+    dy = torch.randn(200, 64, device="cuda").to(dtype)
+
+    def run():
+        for p in moe.parameters():
+            p.grad = None
+        a = x.clone().requires_grad_(True)
+        out = moe(a)
+        out.backward(dy)
+        return [out, a.grad] + [p.grad for p in moe.parameters()]
+
+    assert moe.experts.can_run_layer(x, top_k)
+    whole = run()
+    hook = moe.experts.activation.register_forward_hook(lambda m, i, o: None)
+    assert not moe.experts.can_run_layer(x, top_k)
+    hook.remove()
+    moe.experts.can_run_layer = lambda inp, k: False      # the chain of nodes
+    try:
+        chain = run()
+    finally:
+        del moe.experts.can_run_layer
+    for got, want in zip(whole, chain):
+        assert (got is None) == (want is None)
+        if got is not None:
+            assert torch.equal(got, want)
