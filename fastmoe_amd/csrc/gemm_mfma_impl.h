@@ -343,6 +343,9 @@ constexpr int kXcdRun = 32;
 // column.  32 consecutive numbers are a 4x8 patch (12 operand tiles for 32
 // products), 256 consecutive ones a 16x16 region.  Ragged edges shrink the
 // band, block or patch; the order stays a bijection.
+// (The three sizes can be set at build time, for measurements of other walks:
+// FETCH_SIZE per cfg-4 forward launch was 2.72 GiB with 4 x 8 patches, 2.72 GiB with
+// 8 x 4, 3.88 GiB with 2 x 16 and 4.04 GiB with 16 x 2.)
 #ifndef FMOE_PATCH_ROWS
 #define FMOE_PATCH_ROWS 4
 #define FMOE_PATCH_COLS 8
@@ -1485,6 +1488,9 @@ __device__ __forceinline__ void edge_aware_tile(const GemmArgs& g, uint16_t* sme
 // rather than of its copies (measured on the cfg-2 shapes with +-3 % ragged experts:
 // forward K = 4096 136 -> 128 us, dX K = 4096 151 -> 143 us, fused backward 325 ->
 // 311 us; nothing changes where no narrow tiles run).
+// (Making every remainder tile narrow, whatever their number, was measured and dropped:
+// level on the cfg-2 and cfg-5 shapes, 5-17 % slower on the cfg-3 ones, where 128-row
+// remainders behind capacity-capped experts would stream their rows two or four times.)
 constexpr int kNarrowMax = 128;
 constexpr int kNarrowMinK = 2048;
 constexpr int kNarrowBK = 64;

@@ -16,7 +16,7 @@ from oracle import moe_oracle as O
 
 pytestmark = pytest.mark.gpu
 
-ROW_TOL = 3e-2      # row-wise bound for bf16 results (2e-2 norm-wise)
+ROW_TOL = 2e-2      # row-wise bound for bf16 results, the same as the norm-wise one
 
 
 def _bench_layer(name):
@@ -104,8 +104,8 @@ def test_config4_mixtral_sized_layer_on_a_sample():
     """16384 tokens, d_model 4096, d_hidden 14336, 8 experts, top-2: 23 TFLOP per
     step, too much for the host in full.  The oracle is evaluated on a fixed
     sample of 384 tokens (their outputs and input gradients need nothing else)
-    and on ALL rows of one expert (its four parameter gradients need nothing
-    else); a second expert's bias gradients come from a third, cheap run."""
+    and, expert by expert, on ALL rows of each of the eight experts (an expert's
+    four parameter gradients need nothing but its own rows)."""
     cfg, layer, x, dy = _bench_layer("cfg4")
     out, dx = _run_device(layer, x, dy, detach_score=True)
     with torch.no_grad():
@@ -126,9 +126,9 @@ def test_config4_mixtral_sized_layer_on_a_sample():
     _check("dx[sample]", dx[sample.cuda()], xs.grad)
     del cpu
 
-    # (b) every row of one expert: its slots keep their index (renamed 0), all
-    # other slots are dropped, and the weights handed over are that expert's alone
-    for e, what in ((5, "all"),):
+    # (b) every row of one expert at a time: its slots keep their index (renamed 0),
+    # all other slots are dropped, and the weights handed over are that expert's alone
+    for e in range(cfg["E"]):
         rows = torch.nonzero((idx_c == e).any(dim=1)).view(-1)
         sub_idx = torch.where(idx_c[rows] == e, 0, -1)
         one = _expert_params_cpu(layer, experts=slice(e, e + 1))
