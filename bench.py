@@ -52,19 +52,30 @@ DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 PEAK = {"hbm": 8.0e12, "bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 
 # Bytes per launch (read + write) that leave L2 towards the Infinity Cache and
-# HBM, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script, scaled
-# by what the same counters read in the same run for the row-scatter kernel,
-# whose traffic is known (FETCH_SIZE x 1.035 on cfg2 and cfg5, x 0.998 on cfg4;
-# WRITE_SIZE x 1.000).  Only the workloads that were measured have an entry.
+# HBM, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script
+# (`--counter-pass`; the commands and per-kernel tables are in
+# profiles/moe_step_<config>_hbm_traffic.md), scaled by what the same counters read in
+# the same run for the row-scatter kernel, whose traffic is known: FETCH_SIZE x 0.998
+# on cfg4 and x 1.035 on cfg2 (applied to cfg1, cfg3 and cfg5 as well, whose scatter
+# reads part of its input from L2), WRITE_SIZE x 1.000.  MiB, read + written.  A
+# config without an entry for its dominant op makes the run fail: measure, then add.
+MiB = 2 ** 20
 MEASURED_TRAFFIC = {
-    ("cfg2", "grouped_linear_bwd"): (311.1 + 214.6) * 2 ** 20,       # avg of both layers
-    ("cfg2", "grouped_linear_fwd"): (172.1 + 32.2) * 2 ** 20,
-    ("cfg2", "grouped_linear_fwd_act"): (138.7 + 257.0) * 2 ** 20,
-    ("cfg4", "grouped_linear_bwd"): (5962.0 + 1517.7) * 2 ** 20,     # avg of both layers
-    ("cfg4", "grouped_linear_fwd"): (2927.7 + 258.0) * 2 ** 20,
-    ("cfg4", "grouped_linear_fwd_act"): (2929.8 + 1799.0) * 2 ** 20,
-    ("cfg5", "grouped_linear_bwd"): (1247.1 + 961.3) * 2 ** 20,
-    ("cfg5", "grouped_linear_fwd"): (811.3 + 216.0) * 2 ** 20,
+    ("cfg1", "grouped_linear_bwd"): (2.68 + 1.25) * MiB,             # dX, dW and bias-gradient kernels
+    ("cfg1", "grouped_linear_fwd"): (1.22 + 0.75) * MiB,
+    ("cfg1", "grouped_linear_fwd_act"): (1.22 + 0.75) * MiB,
+    ("cfg2", "grouped_linear_bwd"): (310.9 + 214.6) * MiB,           # avg of both layers
+    ("cfg2", "grouped_linear_fwd"): (172.1 + 32.2) * MiB,
+    ("cfg2", "grouped_linear_fwd_act"): (138.6 + 257.0) * MiB,
+    ("cfg3", "grouped_linear_bwd"): (2103.5 + 2297.3) * MiB,         # avg of both layers
+    ("cfg3", "grouped_linear_fwd"): (1570.1 + 159.4) * MiB,
+    ("cfg3", "grouped_linear_fwd_act"): (1570.1 + 159.4 + 127.2 + 253.3) * MiB,  # + activation kernel
+    ("cfg4", "grouped_linear_bwd"): (6009.1 + 1517.7) * MiB,         # avg of both layers
+    ("cfg4", "grouped_linear_fwd"): (2928.1 + 258.0) * MiB,
+    ("cfg4", "grouped_linear_fwd_act"): (2927.0 + 1799.0) * MiB,
+    ("cfg5", "grouped_linear_bwd"): (1248.4 + 949.7) * MiB,          # avg of both layers
+    ("cfg5", "grouped_linear_fwd"): (815.8 + 217.5) * MiB,
+    ("cfg5", "grouped_linear_fwd_act"): (815.8 + 217.5 + 88.5 + 176.0) * MiB,    # + activation kernel
 }
 
 
@@ -335,6 +346,9 @@ def main():
                          "reference's list of single-expert modules (the kernels then read "
                          "the weights through pointer tables); list implies --no-cpu "
                          "--no-yardstick")
+    ap.add_argument("--counter-pass", action="store_true",
+                    help="for the rocprofv3 runs that measure roofline.traffic themselves: "
+                         "report it as null instead of looking it up")
     ap.add_argument("--no-yardstick", action="store_true",
                     help="skip the untimed torch.mm (hipBLASLt) comparison of the expert GEMMs")
     ap.add_argument("--graph", action="store_true",
@@ -427,8 +441,16 @@ def main():
         roofline = {"kernel": dom, "bound": "hbm", "achieved": round(amount / avg_s / 1e9, 2),
                     "peak": PEAK["hbm"] / 1e9, "unit": "GB/s"}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
-    traffic = MEASURED_TRAFFIC.get((args.config, dom))
-    roofline["traffic"] = None if traffic is None else round(traffic)
+    if args.counter_pass:
+        roofline["traffic"] = None
+    elif (args.config, dom) not in MEASURED_TRAFFIC:
+        # a stale or missing entry must not pass silently as "no data"
+        sys.exit(f"bench.py: no measured HBM traffic on record for {dom} on {args.config}: "
+                 "run the rocprofv3 FETCH_SIZE / WRITE_SIZE passes named in "
+                 f"profiles/moe_step_{args.config}_hbm_traffic.md and add the entry to "
+                 "MEASURED_TRAFFIC")
+    else:
+        roofline["traffic"] = round(MEASURED_TRAFFIC[(args.config, dom)])
     roofline["avg_launch_us"] = kernels[dom]["avg_us"] if hooks else None
 
     result = {
