@@ -79,9 +79,11 @@ Tensor workspace(int64_t numel, int64_t n_expert, const Tensor& like) {
     return torch::empty({bytes}, opts);
   }
   static std::mutex mu;
-  static std::map<std::pair<int, void*>, Tensor> cache;
+  // (never destroyed: at process exit the tensors must not be freed after torch's
+  // allocator has gone)
+  static auto* cache = new std::map<std::pair<int, void*>, Tensor>();
   std::lock_guard<std::mutex> lock(mu);
-  Tensor& ws = cache[{(int)like.device().index(), stream}];
+  Tensor& ws = (*cache)[{(int)like.device().index(), stream}];
   if (!ws.defined() || ws.numel() < bytes) ws = torch::empty({std::max<int64_t>(bytes, 1 << 16)}, opts);
   return ws;
 }
