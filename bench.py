@@ -10,7 +10,12 @@ already resident in HBM.  Prints ONE JSON line:
   roofline            the kernel that takes the most time in a step: achieved
                       algorithmic FLOP/s (or bytes/s) per launch, from HIP
                       events recorded around every launch inside the timed
-                      region on the stream the kernels run on
+                      region on the stream the kernels run on.  A grouped GEMM
+                      is priced against the roofline its own arithmetic puts
+                      it under: HBM when every operand and result moved once
+                      at 8 TB/s takes longer than its FLOPs at the matrix
+                      cores' peak (many short experts on large weights),
+                      else MFMA; the other fraction rides along
   cpu_baseline        the CPU checker's brute-force layer (torch fp32 on the
                       host cores) timed on a bounded sample of the same workload
   kernels             per-kernel average time and achieved rate, from an untimed
@@ -222,6 +227,26 @@ def kernel_work(cfg: dict, n_valid: int):
     }
 
 
+def gemm_bytes(cfg: dict, n_valid: int, e_live: int):
+    """Algorithmic HBM bytes of ONE launch of each grouped GEMM: every operand and
+    result once.  Experts without rows have no tiles in the forward and dX products
+    (their weights are not read); dW writes every expert's gradient, zeros included.
+    A workload of many short experts (cfg3: 64 experts of 62-640 rows on 32 MiB
+    weights) moves more bytes per FLOP than the matrix-core roofline's ridge, and is
+    then to be read against the HBM roofline."""
+    d, h, E = cfg["d"], cfg["h"], cfg["E"]
+    s = 4 if cfg["dtype"] == "f32" else 2
+    rows = n_valid * (d + h) * s          # one activation operand + one result, avg of both layers
+    w_live, w_all = e_live * d * h * s, E * d * h * s
+    return {
+        "grouped_linear_fwd": rows + w_live,
+        "grouped_linear_fwd_act": rows + n_valid * h * s + w_live,     # second result: gelu
+        "grouped_linear_dgrad": rows + w_live,
+        "grouped_linear_wgrad": rows + w_all,
+        "grouped_linear_bwd": 1.5 * rows + w_live + w_all,             # dy, x read; dx written
+    }
+
+
 def cpu_baseline(cfg: dict, layer, x, target_seconds: float = 15.0):
     """The CPU checker's brute-force layer (fp32, all host threads) on the first
     S tokens of the workload, S sized for about `target_seconds` of work."""
@@ -378,6 +403,8 @@ def main():
         idx, _ = layer.gate(x)
     n_valid = int((idx >= 0).sum().item())
     work = kernel_work(cfg, n_valid)
+    e_live = int(torch.bincount(idx[idx >= 0].flatten(), minlength=cfg["E"]).ne(0).sum().item())
+    gbytes = gemm_bytes(cfg, n_valid, e_live)
 
     def summarise(records, n_steps):
         per = {}
@@ -399,6 +426,9 @@ def main():
                     round(rate / (1e12 if kind == "flop" else 1e9), 2),
                 "frac_of_peak": round(rate / peak, 4),
             }
+            if name in gbytes and avg_ms > 0:
+                out[name]["hbm_frac_of_peak"] = round(
+                    gbytes[name] / (avg_ms * 1e-3) / PEAK["hbm"], 4)
         return out
 
     # Untimed survey pass with an event pair around every op: the per-kernel
@@ -434,9 +464,16 @@ def main():
         kernels[dom] = dict(timed[dom], timed_region=True)
     kind, amount = work[dom] if hooks else ("flop", 0.0)
     avg_s = kernels[dom]["avg_us"] * 1e-6 if hooks else 1.0
-    if kind == "flop":
+    if kind == "flop" and gbytes.get(dom, 0.0) / PEAK["hbm"] > amount / PEAK[cfg["dtype"]]:
+        # more HBM time than matrix-core time in the algorithm itself: memory roofline
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": round(gbytes[dom] / avg_s / 1e9, 2),
+                    "peak": PEAK["hbm"] / 1e9, "unit": "GB/s",
+                    "mfma_frac": round(amount / avg_s / PEAK[cfg["dtype"]], 4)}
+    elif kind == "flop":
         roofline = {"kernel": dom, "bound": "mfma", "achieved": round(amount / avg_s / 1e12, 2),
                     "peak": PEAK[cfg["dtype"]] / 1e12, "unit": "TFLOP/s"}
+        if dom in gbytes:
+            roofline["hbm_frac"] = round(gbytes[dom] / avg_s / PEAK["hbm"], 4)
     else:
         roofline = {"kernel": dom, "bound": "hbm", "achieved": round(amount / avg_s / 1e9, 2),
                     "peak": PEAK["hbm"] / 1e9, "unit": "GB/s"}

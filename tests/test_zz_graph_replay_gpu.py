@@ -59,3 +59,37 @@ def test_forward_and_backward_replay_from_a_hip_graph():
             assert torch.equal(a, b)
         _ = eager(xs[(i + 1) % 4], dys[(i + 1) % 4])   # eager work between replays
         torch.cuda.synchronize()
+
+
+def test_make_graphed_callables_replays_the_layer():
+    """torch.cuda.make_graphed_callables captures the layer's forward and backward in
+    two graphs behind an ordinary autograd interface.  The graphed layer gives the
+    bits of an eager twin on new data with other routings, with eager work and
+    synchronisations between its calls."""
+    import copy
+
+    dtype = torch.bfloat16
+    moe = _make(8, 128, 256, 2, dtype, seed=5, scale=0.05)
+    twin = copy.deepcopy(moe)
+    g = torch.Generator().manual_seed(22)
+    xs = [torch.randn(300, 128, generator=g).to(dtype).cuda() for _ in range(4)]
+    dys = [torch.randn(300, 128, generator=g).to(dtype).cuda() for _ in range(4)]
+
+    def run(layer, x, dy):
+        params = list(layer.parameters())
+        for p in params:
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        out = layer(xi)
+        out.backward(dy)
+        return [out.detach().clone(), xi.grad.clone()] + [p.grad.clone() for p in params]
+
+    want = [run(twin, x, dy) for x, dy in zip(xs, dys)]
+    graphed = torch.cuda.make_graphed_callables(moe, (xs[0].clone().requires_grad_(True),))
+    for i in (1, 2, 3, 0, 2):
+        got = run(graphed, xs[i], dys[i])
+        torch.cuda.synchronize()
+        for a, b in zip(got, want[i]):
+            assert torch.equal(a, b)
+        _ = run(twin, xs[(i + 1) % 4], dys[(i + 1) % 4])
+        torch.cuda.synchronize()
