@@ -104,16 +104,20 @@ def test_compiled_module_matches_the_ctypes_module_bit_for_bit():
 
 @pytest.mark.gpu
 @pytest.mark.timeout(900)
-def test_suites_pass_on_the_ctypes_binding():
+@pytest.mark.parametrize("suites", [
+    ("tests/test_routing_gpu.py", "tests/test_dispatch_gpu.py", "tests/test_act_gpu.py"),
+    ("tests/test_linear_gpu.py",),
+    ("tests/test_layer_gpu.py", "tests/test_fused_act_gpu.py"),
+], ids=["routing-dispatch-act", "linear", "layer-fused_act"])
+def test_suites_pass_on_the_ctypes_binding(suites):
     """Routing, dispatch, linear, activation and layer suites with the package bound
-    to the ctypes calls instead of the compiled extension (one child process; the big
-    benchmark-size cases stay with the default binding).  The activation suites also
-    watch the per-op event hook, which both bindings must feed alike."""
+    to the ctypes calls instead of the compiled extension (one child process per group of
+    suites, so that none runs for minutes without a sign of life; the big benchmark-size
+    cases stay with the default binding).  The activation suites also watch the per-op
+    event hook, which both bindings must feed alike."""
     env = dict(os.environ, FMOE_BINDING="ctypes")
     cmd = [sys.executable, "-m", "pytest", "-x", "-q", "-m", "gpu", "-p", "no:cacheprovider",
-           "tests/test_routing_gpu.py", "tests/test_dispatch_gpu.py", "tests/test_linear_gpu.py",
-           "tests/test_layer_gpu.py", "tests/test_act_gpu.py", "tests/test_fused_act_gpu.py",
-           "-k", "not full_size and not config2"]
+           *suites, "-k", "not full_size and not config2"]
     res = subprocess.run(cmd, cwd=ROOT, env=env, capture_output=True, text=True, timeout=850)
     tail = (res.stdout + res.stderr)[-3000:]
     assert res.returncode == 0, tail
