@@ -62,11 +62,13 @@ def test_forward_and_backward_replay_from_a_hip_graph():
 
 
 def test_make_graphed_callables_replays_the_layer():
-    """torch.cuda.make_graphed_callables captures the layer's forward and backward in
-    two graphs behind an ordinary autograd interface.  The graphed layer gives the
-    bits of an eager twin on new data with other routings, with eager work and
-    synchronisations between its calls."""
+    """fastmoe_amd.graphed (torch.cuda.make_graphed_callables behind the library's
+    set-up) captures the layer's forward and backward in two graphs behind an ordinary
+    autograd interface.  The graphed layer gives the bits of an eager twin on new data
+    with other routings, with eager work and synchronisations between its calls."""
     import copy
+
+    import fastmoe_amd
 
     dtype = torch.bfloat16
     moe = _make(8, 128, 256, 2, dtype, seed=5, scale=0.05)
@@ -85,7 +87,7 @@ def test_make_graphed_callables_replays_the_layer():
         return [out.detach().clone(), xi.grad.clone()] + [p.grad.clone() for p in params]
 
     want = [run(twin, x, dy) for x, dy in zip(xs, dys)]
-    graphed = torch.cuda.make_graphed_callables(moe, (xs[0].clone().requires_grad_(True),))
+    graphed = fastmoe_amd.graphed(moe, xs[0].clone().requires_grad_(True))
     for i in (1, 2, 3, 0, 2):
         got = run(graphed, xs[i], dys[i])
         torch.cuda.synchronize()
