@@ -7,6 +7,12 @@
 // read against it.  The 2 GiB source is eight times the last-level cache; the 256 MiB
 // run shows the same loops when the data stays in that cache.
 //
+// A second set of loops only stores: 256 x 256 tiles of 2-byte elements (256 row
+// segments of 512 bytes at the row pitch of a gradient matrix, every thread one 16-byte
+// pack of every eighth row: the store pattern of the grouped GEMM's output tiles), one
+// tile per workgroup, against the same bytes stored as one 128 KiB run per workgroup.
+// They give the time below which no kernel that writes such tiles can go.
+//
 //   hipcc --offload-arch=gfx950 -O3 tests/hbm_probe.hip -o /tmp/hbm_probe && /tmp/hbm_probe
 #include <hip/hip_runtime.h>
 
@@ -62,6 +68,45 @@ __global__ void __launch_bounds__(256) mover(const pack_t* __restrict__ src,
     for (int u = 1; u < U; ++u) a ^= acc[u];
     if (a.x == 0x12345678u && a.y == 0x9abcdef0u && a.z == 77u) dst[lane] = a;
   }
+}
+
+// One workgroup stores one tile: tiles_n tiles side by side, pitch = tiles_n * 512 bytes
+// (tiles_n == 0: the tile as one run of 128 KiB).
+__global__ void __launch_bounds__(256) tile_writer(char* __restrict__ dst, int tiles_n,
+                                                   long pitch) {
+  const int tid = threadIdx.x, pk = tid % 32, r0 = tid / 32;
+  const long t = blockIdx.x;
+  char* base = tiles_n == 0 ? dst + t * 131072
+                            : dst + (t / tiles_n) * 256 * pitch + (t % tiles_n) * 512;
+  const long row_bytes = tiles_n == 0 ? 512 : pitch;
+  const pack_t v = {(unsigned)tid, (unsigned)t, 7u, 9u};
+#pragma unroll
+  for (int u = 0; u < 32; ++u)
+    *reinterpret_cast<pack_t*>(base + (long)(u * 8 + r0) * row_bytes + pk * 16) = v;
+}
+
+static void run_tiles(const char* what, char* dst, long dst_bytes, int tiles_n) {
+  const long pitch = tiles_n == 0 ? 512 : (long)tiles_n * 512;
+  const long tiles = dst_bytes / 131072;
+  // whole rows of tiles only, and nothing past the allocation
+  if (tiles_n != 0 && tiles % tiles_n != 0) { printf("tile grid does not fit\n"); exit(1); }
+  const long last = tiles_n == 0 ? tiles * 131072 : (tiles / tiles_n) * 256 * pitch;
+  if (last > dst_bytes) { printf("tile grid past the allocation\n"); exit(1); }
+  hipEvent_t a, b;
+  CK(hipEventCreate(&a));
+  CK(hipEventCreate(&b));
+  for (int i = 0; i < 3; ++i) tile_writer<<<(int)tiles, 256>>>(dst, tiles_n, pitch);
+  CK(hipEventRecord(a));
+  const int iters = 20;
+  for (int i = 0; i < iters; ++i) tile_writer<<<(int)tiles, 256>>>(dst, tiles_n, pitch);
+  CK(hipEventRecord(b));
+  CK(hipEventSynchronize(b));
+  float ms;
+  CK(hipEventElapsedTime(&ms, a, b));
+  const double us = ms * 1e3 / iters;
+  printf("| %-40s | %5ld | %8.1f | %5.2f | %.3f | %5.2f |\n", what, tiles, us,
+         tiles * 131072.0 / us * 1e-6, tiles * 131072.0 / us * 1e-6 / 8.0, us / (tiles / 256.0));
+  fflush(stdout);
 }
 
 template <int U, int R, int W>
@@ -121,5 +166,11 @@ int main() {
     run<4, 3, 2>("permuted 4 KiB, 3 reads per 2 writes (combine bwd)", src, idx, dst, bytes);
     run<4, 8, 1>("permuted 4 KiB, 8 reads per write (combine k=8)", src, idx, dst, bytes);
   }
+  printf("\nstores only, 256 x 256 tiles of 2-byte elements, one tile per workgroup\n\n");
+  printf("| pattern | tiles | us | TB/s | of 8 TB/s | us per round of 256 tiles |\n|---|---|---|---|---|---|\n");
+  run_tiles("128 KiB runs", (char*)dst, big, 0);
+  run_tiles("tile rows at a pitch of 16 KiB (8192 columns)", (char*)dst, big, 32);
+  run_tiles("tile rows at a pitch of 4 KiB (2048 columns)", (char*)dst, big, 8);
+  run_tiles("tile rows at a pitch of 8 KiB (4096 columns)", (char*)dst, big, 16);
   return 0;
 }
